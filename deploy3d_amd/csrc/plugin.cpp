@@ -1,0 +1,754 @@
+// Host side of the engine: the two plugin objects behind the C ABI of
+// include/d3d_spconv.h, attribute-blob parsing, weight preparation, and the
+// per-index-tensor cache of neighbour tables that implements indice-key reuse.
+//
+// Reference life cycle being mirrored: SPConvIdxPlugin (trt/spconv/index_trt.cu:52-249)
+// and SPConvMMPlugin (trt/spconv/mm_trt.cu:39-206).
+#include <cmath>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <new>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+namespace d3d {
+
+// ---------------------------------------------------------------------------
+// error text (thread local)
+// ---------------------------------------------------------------------------
+namespace {
+thread_local char g_error[512] = "";
+}
+
+void setError(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+const char* lastError() { return g_error; }
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// device memory
+// ---------------------------------------------------------------------------
+struct DeviceBuffer {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  DeviceBuffer() = default;
+  DeviceBuffer(const DeviceBuffer&) = delete;
+  DeviceBuffer& operator=(const DeviceBuffer&) = delete;
+  ~DeviceBuffer() {
+    if (ptr) (void)hipFree(ptr);
+  }
+  int32_t reserve(size_t n) {
+    if (n <= bytes) return D3D_OK;
+    if (ptr) {
+      D3D_HIP_CHECK(hipFree(ptr));
+      ptr = nullptr;
+      bytes = 0;
+    }
+    D3D_HIP_CHECK(hipMalloc(&ptr, n));
+    bytes = n;
+    return D3D_OK;
+  }
+  int32_t upload(const void* src, size_t n) {
+    int32_t rc = reserve(n);
+    if (rc != D3D_OK) return rc;
+    D3D_HIP_CHECK(hipMemcpy(ptr, src, n, hipMemcpyHostToDevice));
+    return D3D_OK;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// IEEE conversions on the host (round-to-nearest-even), written out so the
+// library does not depend on the host compiler's _Float16 runtime support.
+// ---------------------------------------------------------------------------
+uint16_t floatToHalfBits(float f) {
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  x &= 0x7FFFFFFFu;
+  if (x >= 0x7F800000u) return static_cast<uint16_t>(sign | 0x7C00u | (x > 0x7F800000u ? 0x200u : 0));  // inf / nan
+  if (x >= 0x477FF000u) return static_cast<uint16_t>(sign | 0x7C00u);  // rounds to >= 65520 -> inf
+  if (x < 0x33000001u) return static_cast<uint16_t>(sign);             // below half of the smallest subnormal
+  int exp = static_cast<int>(x >> 23) - 127;
+  uint32_t man = (x & 0x7FFFFFu) | 0x800000u;
+  int shift;
+  uint32_t base;
+  if (exp < -14) {  // subnormal half
+    shift = 13 + (-14 - exp);
+    base = 0;
+  } else {
+    shift = 13;
+    base = static_cast<uint32_t>(exp + 15) << 10;
+    man &= 0x7FFFFFu;
+  }
+  uint32_t q = man >> shift;
+  const uint32_t rem = man & ((1u << shift) - 1), half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (q & 1))) ++q;
+  return static_cast<uint16_t>(sign | (base + q));  // a mantissa carry correctly bumps the exponent
+}
+
+float halfBitsToFloat(uint16_t h) {
+  const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
+  const uint32_t exp = (h >> 10) & 0x1F, man = h & 0x3FFu;
+  uint32_t x;
+  if (exp == 0) {
+    if (man == 0) {
+      x = sign;
+    } else {
+      float v = std::ldexp(static_cast<float>(man), -24);
+      std::memcpy(&x, &v, 4);
+      x |= sign;
+    }
+  } else if (exp == 31) {
+    x = sign | 0x7F800000u | (man << 13);
+  } else {
+    x = sign | ((exp + 112) << 23) | (man << 13);
+  }
+  float f;
+  std::memcpy(&f, &x, 4);
+  return f;
+}
+
+uint16_t floatToBf16Bits(float f) {
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  if ((x & 0x7FFFFFFFu) > 0x7F800000u) return static_cast<uint16_t>((x >> 16) | 0x40u);  // quiet nan
+  x += 0x7FFFu + ((x >> 16) & 1u);
+  return static_cast<uint16_t>(x >> 16);
+}
+
+float bf16BitsToFloat(uint16_t b) {
+  const uint32_t x = static_cast<uint32_t>(b) << 16;
+  float f;
+  std::memcpy(&f, &x, 4);
+  return f;
+}
+
+int dtypeBytes(int32_t dtype) {
+  switch (dtype) {
+    case D3D_FLOAT:
+    case D3D_INT32: return 4;
+    case D3D_HALF:
+    case D3D_BF16: return 2;
+    case D3D_INT8:
+    case D3D_BOOL: return 1;
+  }
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// neighbour-table cache: one entry per index tensor (the value an indice key
+// names in the calling graph).  The rulebook operator bumps the generation of
+// its output tensor; the first convolution that consumes a generation builds
+// the table, the other convolutions sharing the key reuse it.  An index
+// tensor this library did not produce has no generation to trust, so its
+// table is rebuilt on every convolution.
+// ---------------------------------------------------------------------------
+struct NbrTable {
+  std::shared_ptr<DeviceBuffer> buf;
+  uint64_t builtGeneration = 0;
+  bool built = false;
+  int kVol = 0;
+  int64_t outRows = 0, rowLen = 0;
+  const void* numIndex = nullptr;
+};
+struct NbrEntry {
+  bool managed = false;
+  uint64_t generation = 0;
+  NbrTable forward, inverse;
+};
+std::mutex g_cacheMutex;
+std::unordered_map<const void*, NbrEntry> g_cache;
+
+void noteRulebookWritten(const void* index) {
+  std::lock_guard<std::mutex> lock(g_cacheMutex);
+  NbrEntry& e = g_cache[index];
+  e.managed = true;
+  ++e.generation;
+}
+
+int32_t neighbourTable(const int32_t* index, int64_t rowLen, const int32_t* numIndex, bool inverse, int kVol,
+                       int64_t outRows, hipStream_t stream, std::shared_ptr<DeviceBuffer>* out) {
+  std::lock_guard<std::mutex> lock(g_cacheMutex);
+  NbrEntry& e = g_cache[index];
+  NbrTable& t = inverse ? e.inverse : e.forward;
+  const bool fresh = e.managed && t.built && t.builtGeneration == e.generation && t.kVol == kVol &&
+                     t.outRows == outRows && t.rowLen == rowLen && t.numIndex == numIndex;
+  if (!fresh) {
+    const size_t bytes = static_cast<size_t>(kVol) * static_cast<size_t>(outRows) * sizeof(int32_t);
+    if (!t.buf || t.buf->bytes < bytes) {
+      auto nb = std::make_shared<DeviceBuffer>();
+      int32_t rc = nb->reserve(bytes > 0 ? bytes : 4);
+      if (rc != D3D_OK) return rc;
+      t.buf = nb;  // an older table stays alive while an enqueued kernel's owner still holds it
+    }
+    int32_t rc = launchBuildNeighbours(index, rowLen, numIndex, inverse, kVol, outRows,
+                                       static_cast<int32_t*>(t.buf->ptr), stream);
+    if (rc != D3D_OK) return rc;
+    t.built = true;
+    t.builtGeneration = e.generation;
+    t.kVol = kVol;
+    t.outRows = outRows;
+    t.rowLen = rowLen;
+    t.numIndex = numIndex;
+  }
+  *out = t.buf;
+  return D3D_OK;
+}
+
+// ---------------------------------------------------------------------------
+// packed little-endian blob reader
+// (reference: SerializeStream, trt/include/common/refnd.h:258-294)
+// ---------------------------------------------------------------------------
+struct BlobReader {
+  const uint8_t* p;
+  size_t len, pos = 0;
+  BlobReader(const void* data, size_t n) : p(static_cast<const uint8_t*>(data)), len(n) {}
+  bool i32(int32_t* v) {
+    if (pos + 4 > len) return false;
+    std::memcpy(v, p + pos, 4);
+    pos += 4;
+    return true;
+  }
+  bool u8(uint8_t* v) {
+    if (pos + 1 > len) return false;
+    *v = p[pos++];
+    return true;
+  }
+};
+
+}  // namespace
+}  // namespace d3d
+
+// ---------------------------------------------------------------------------
+// plugin objects
+// ---------------------------------------------------------------------------
+struct d3d_plugin {
+  std::string type;
+  std::vector<uint8_t> blob;  // kept verbatim: serialize() is a byte-exact round trip
+  virtual ~d3d_plugin() = default;
+  virtual d3d_plugin* clone() const = 0;
+  virtual int32_t numOutputs() const = 0;
+  virtual int32_t outputDims(int32_t idx, const d3d_tensor_desc* in, int32_t nbIn, d3d_tensor_desc* out) const = 0;
+  virtual int32_t outputDtype(int32_t idx, const int32_t* inTypes, int32_t nbIn) const = 0;
+  virtual int32_t supportsFormat(int32_t pos, const d3d_tensor_desc* io, int32_t nbIn, int32_t nbOut) const = 0;
+  virtual int32_t configure(const d3d_tensor_desc* in, int32_t nbIn, const d3d_tensor_desc* out, int32_t nbOut) = 0;
+  virtual size_t workspaceSize(const d3d_tensor_desc* in, int32_t nbIn) const = 0;
+  virtual int32_t enqueue(const d3d_tensor_desc* inDesc, const d3d_tensor_desc* outDesc, const void* const* inputs,
+                          void* const* outputs, void* workspace, size_t workspaceBytes, hipStream_t stream) = 0;
+};
+
+namespace d3d {
+namespace {
+
+// --- SPConvIdx{N}d -----------------------------------------------------------
+// Attribute layout: SPConvIdxPluginParam<NDim>, trt/spconv/index_trt.cu:39-50.
+struct IdxPlugin final : d3d_plugin {
+  int nd = 3;
+  int32_t kernel[kMaxSpatial], stride[kMaxSpatial], padding[kMaxSpatial], dilation[kMaxSpatial],
+      outPadding[kMaxSpatial];
+  int32_t maxNumActOut = 0;
+  bool subM = false, transpose = false;
+
+  int kVol() const {
+    int v = 1;
+    for (int i = 0; i < nd; ++i) v *= kernel[i];
+    return v;
+  }
+
+  static int32_t parse(int nd, const void* data, size_t len, IdxPlugin** out) {
+    const size_t need = static_cast<size_t>(nd) * 5 * 4 + 4 + 2;
+    if (!data || len < need) {
+      setError("SPConvIdx%dd: attribute blob of %zu bytes, %zu expected", nd, len, need);
+      return D3D_ERR_BAD_BLOB;
+    }
+    auto p = std::unique_ptr<IdxPlugin>(new IdxPlugin());
+    p->nd = nd;
+    p->type = "SPConvIdx" + std::to_string(nd) + "d";
+    BlobReader r(data, len);
+    int32_t* fields[5] = {p->kernel, p->stride, p->padding, p->dilation, p->outPadding};
+    for (auto* f : fields)
+      for (int i = 0; i < nd; ++i) r.i32(&f[i]);
+    r.i32(&p->maxNumActOut);
+    uint8_t b0 = 0, b1 = 0;
+    r.u8(&b0);
+    r.u8(&b1);
+    p->subM = b0 != 0;
+    p->transpose = b1 != 0;
+    for (int i = 0; i < nd; ++i) {
+      if (p->kernel[i] < 1 || p->stride[i] < 1 || p->dilation[i] < 1 || p->padding[i] < 0) {
+        setError("%s: kernel/stride/dilation must be positive and padding non-negative", p->type.c_str());
+        return D3D_ERR_BAD_BLOB;
+      }
+    }
+    if (p->maxNumActOut < 0) {
+      setError("%s: negative maxNumActOut", p->type.c_str());
+      return D3D_ERR_BAD_BLOB;
+    }
+    p->blob.assign(static_cast<const uint8_t*>(data), static_cast<const uint8_t*>(data) + need);
+    *out = p.release();
+    return D3D_OK;
+  }
+
+  d3d_plugin* clone() const override { return new IdxPlugin(*this); }
+  int32_t numOutputs() const override { return subM ? 2 : 5; }  // index_trt.cu:98-101
+
+  // spatial extents of the output grid from those of the input grid
+  void outSpatial(const int32_t* in, int32_t* out) const {
+    for (int i = 0; i < nd; ++i) {
+      if (transpose) {  // geometry.h:138-156
+        out[i] = (in[i] - 1) * stride[i] - 2 * padding[i] + (kernel[i] - 1) * dilation[i] + outPadding[i] + 1;
+      } else {  // geometry.h:118-136
+        out[i] = (in[i] + 2 * padding[i] - dilation[i] * (kernel[i] - 1) - 1) / stride[i] + 1;
+      }
+    }
+  }
+
+  int32_t outputDims(int32_t idx, const d3d_tensor_desc* in, int32_t nbIn, d3d_tensor_desc* out) const override {
+    if (!in || nbIn < 3 || !out || idx < 0 || idx >= numOutputs()) {
+      setError("%s: output %d of %d, %d inputs", type.c_str(), idx, numOutputs(), nbIn);
+      return D3D_ERR_BAD_ARG;
+    }
+    std::memset(out, 0, sizeof(*out));
+    out->dtype = D3D_INT32;
+    out->format = D3D_LINEAR;
+    switch (idx) {
+      case 0:  // index_trt.cu:107-119
+        out->nb_dims = 2;
+        out->dims[0] = 3;
+        out->dims[1] = kVol() * (in[0].dims[0] + kSegment);
+        break;
+      case 1:
+      case 3:
+        out->nb_dims = 1;
+        out->dims[0] = 1;
+        break;
+      case 2:  // index_trt.cu:123-126
+        out->nb_dims = 2;
+        out->dims[0] = maxNumActOut;
+        out->dims[1] = nd + 1;
+        break;
+      default: {  // index_trt.cu:131-150: [B, 0, spatial...]
+        if (in[2].nb_dims != nd + 2) {
+          setError("%s: spatial-shape tensor must have %d dims", type.c_str(), nd + 2);
+          return D3D_ERR_BAD_ARG;
+        }
+        *out = in[2];
+        out->dtype = D3D_INT32;
+        outSpatial(in[2].dims + 2, out->dims + 2);
+      }
+    }
+    return D3D_OK;
+  }
+  int32_t outputDtype(int32_t, const int32_t*, int32_t) const override { return D3D_INT32; }  // index_trt.cu:153-155
+  int32_t supportsFormat(int32_t pos, const d3d_tensor_desc* io, int32_t nbIn, int32_t nbOut) const override {
+    if (!io || pos < 0 || pos >= nbIn + nbOut) return 0;
+    return io[pos].format == D3D_LINEAR && io[pos].dtype == D3D_INT32;  // index_trt.cu:156-161
+  }
+  int32_t configure(const d3d_tensor_desc*, int32_t, const d3d_tensor_desc*, int32_t) override { return D3D_OK; }
+
+  RbGeom geometry(const int32_t* outGrid /* [B, spatial...] */) const {
+    RbGeom g{};
+    g.nd = nd;
+    const int pad = kMaxSpatial - nd;
+    for (int i = 0; i < kMaxSpatial; ++i) {
+      const bool real = i >= pad;
+      g.k[i] = real ? kernel[i - pad] : 1;
+      g.s[i] = real ? stride[i - pad] : 1;
+      g.p[i] = real ? padding[i - pad] : 0;
+      g.d[i] = real ? dilation[i - pad] : 1;
+      g.shape[i + 1] = real ? outGrid[1 + i - pad] : 1;
+    }
+    g.shape[0] = outGrid[0];
+    g.kVol = kVol();
+    g.transpose = transpose ? 1 : 0;
+    return g;
+  }
+
+  size_t workspaceSize(const d3d_tensor_desc* in, int32_t nbIn) const override {
+    if (!in || nbIn < 1) return 0;
+    int32_t ones[kMaxSpatial + 1] = {1, 1, 1, 1, 1};
+    RbGeom g = geometry(ones);
+    // the grid only caps the strided hash; size for the capacity bound alone
+    for (int i = 0; i <= kMaxSpatial; ++i) g.shape[i] = 1 << 6;
+    return planRulebookWorkspace(g, in[0].dims[0], subM).total;
+  }
+
+  int32_t enqueue(const d3d_tensor_desc* inDesc, const d3d_tensor_desc* outDesc, const void* const* inputs,
+                  void* const* outputs, void* workspace, size_t workspaceBytes, hipStream_t stream) override {
+    if (!inDesc || !outDesc || !inputs || !outputs) {
+      setError("%s: null descriptor or tensor array", type.c_str());
+      return D3D_ERR_BAD_ARG;
+    }
+    if (inDesc[0].nb_dims != 2 || inDesc[0].dims[1] != nd + 1 || inDesc[2].nb_dims != nd + 2) {
+      setError("%s: inCoors must be [cap, %d] and the spatial shape [B, 0, %d extents]", type.c_str(), nd + 1, nd);
+      return D3D_ERR_BAD_ARG;
+    }
+    const int64_t cap = inDesc[0].dims[0];
+    const int64_t rowLen = static_cast<int64_t>(kVol()) * (cap + kSegment);
+    if (outDesc[0].nb_dims != 2 || outDesc[0].dims[0] != 3 || outDesc[0].dims[1] != rowLen) {
+      setError("%s: index tensor must be [3, %lld]", type.c_str(), static_cast<long long>(rowLen));
+      return D3D_ERR_BAD_ARG;
+    }
+    // output grid: the input's for SubM (index_trt.cu:218-219), else derived from it
+    int32_t grid[kMaxSpatial + 1];
+    grid[0] = inDesc[2].dims[0];
+    if (subM) {
+      for (int i = 0; i < nd; ++i) grid[1 + i] = inDesc[2].dims[2 + i];
+    } else {
+      outSpatial(inDesc[2].dims + 2, grid + 1);
+      if (outDesc[2].nb_dims != 2 || outDesc[2].dims[0] != maxNumActOut || outDesc[2].dims[1] != nd + 1) {
+        setError("%s: outCoors must be [%d, %d]", type.c_str(), maxNumActOut, nd + 1);
+        return D3D_ERR_BAD_ARG;
+      }
+    }
+    const RbGeom g = geometry(grid);
+    int32_t rc = launchRulebook(g, subM, static_cast<const int32_t*>(inputs[0]),
+                                static_cast<const int32_t*>(inputs[1]), cap, maxNumActOut,
+                                static_cast<int32_t*>(outputs[0]), static_cast<int32_t*>(outputs[1]),
+                                subM ? nullptr : static_cast<int32_t*>(outputs[2]),
+                                subM ? nullptr : static_cast<int32_t*>(outputs[3]), workspace, workspaceBytes, stream);
+    if (rc == D3D_OK) noteRulebookWritten(outputs[0]);
+    return rc;
+  }
+};
+
+// --- SPConvMM ----------------------------------------------------------------
+// Attribute layout: SPConvMMPluginParam + fp32 payload, trt/spconv/mm_trt.cu:27-37, :61-68.
+constexpr uint32_t kExtMagic = 0x58443344u;  // "D3DX"
+constexpr size_t kMMHeader = 19;
+
+struct MMDeviceWeights {
+  int32_t dtype = -1;
+  DeviceBuffer f32, mfma, bias;
+};
+
+struct MMPlugin final : d3d_plugin {
+  int32_t kernelVol = 0, cin = 0, cout = 0, maxNumActOut = 0;
+  bool inverse = false, withBias = false, relu = false;
+  float actScaleIn = 1.f, actScaleOut = 1.f;
+  size_t weightOffset = kMMHeader;             // byte offset of W in blob
+  std::shared_ptr<MMDeviceWeights> dev;        // shared by clones (mm_trt.cu:43-45, :75-79)
+  std::shared_ptr<std::mutex> devMutex;
+  std::shared_ptr<DeviceBuffer> lastTable;     // keeps the table of the last enqueue alive
+
+  static int32_t parse(const void* data, size_t len, MMPlugin** out) {
+    if (!data || len < kMMHeader) {
+      setError("SPConvMM: attribute blob of %zu bytes, at least %zu expected", len, kMMHeader);
+      return D3D_ERR_BAD_BLOB;
+    }
+    auto p = std::unique_ptr<MMPlugin>(new MMPlugin());
+    p->type = "SPConvMM";
+    BlobReader r(data, len);
+    r.i32(&p->kernelVol);
+    r.i32(&p->cin);
+    r.i32(&p->cout);
+    r.i32(&p->maxNumActOut);
+    uint8_t subM = 0, inv = 0, wb = 0;
+    r.u8(&subM);  // deprecated, ignored (mm_trt.cu:33)
+    r.u8(&inv);
+    r.u8(&wb);
+    p->inverse = inv != 0;
+    p->withBias = wb != 0;
+    if (p->kernelVol < 1 || p->cin < 1 || p->cout < 1 || p->maxNumActOut < 0) {
+      setError("SPConvMM: kernelVol/inChannels/outChannels must be positive");
+      return D3D_ERR_BAD_BLOB;
+    }
+    const size_t floats = static_cast<size_t>(p->kernelVol) * p->cin * p->cout + (p->withBias ? p->cout : 0);
+    const size_t payloadEnd = kMMHeader + floats * 4;
+    if (len < payloadEnd) {
+      setError("SPConvMM: blob holds %zu payload bytes, %zu needed for W[%d,%d,%d]%s", len - kMMHeader, floats * 4,
+               p->kernelVol, p->cin, p->cout, p->withBias ? " + bias" : "");
+      return D3D_ERR_BAD_BLOB;
+    }
+    if (len >= payloadEnd + 20) {  // optional extension record
+      const uint8_t* e = static_cast<const uint8_t*>(data) + payloadEnd;
+      uint32_t magic, version, flags;
+      std::memcpy(&magic, e, 4);
+      std::memcpy(&version, e + 4, 4);
+      std::memcpy(&flags, e + 8, 4);
+      if (magic == kExtMagic) {
+        if (version != 1) {
+          setError("SPConvMM: extension record version %u not understood", version);
+          return D3D_ERR_BAD_BLOB;
+        }
+        p->relu = (flags & 1u) != 0;
+        std::memcpy(&p->actScaleIn, e + 12, 4);
+        std::memcpy(&p->actScaleOut, e + 16, 4);
+      }
+    }
+    p->blob.assign(static_cast<const uint8_t*>(data), static_cast<const uint8_t*>(data) + len);
+    p->dev = std::make_shared<MMDeviceWeights>();
+    p->devMutex = std::make_shared<std::mutex>();
+    *out = p.release();
+    return D3D_OK;
+  }
+
+  d3d_plugin* clone() const override { return new MMPlugin(*this); }
+  int32_t numOutputs() const override { return 1; }
+  int32_t outputDims(int32_t idx, const d3d_tensor_desc*, int32_t, d3d_tensor_desc* out) const override {
+    if (idx != 0 || !out) return D3D_ERR_BAD_ARG;
+    std::memset(out, 0, sizeof(*out));  // mm_trt.cu:98-103
+    out->format = D3D_LINEAR;
+    out->nb_dims = 2;
+    out->dims[0] = maxNumActOut;
+    out->dims[1] = cout;
+    return D3D_OK;
+  }
+  int32_t outputDtype(int32_t, const int32_t* inTypes, int32_t nbIn) const override {
+    return (inTypes && nbIn > 0) ? inTypes[0] : D3D_ERR_BAD_ARG;  // mm_trt.cu:104-106
+  }
+  static bool featureType(int32_t t) { return t == D3D_HALF || t == D3D_FLOAT || t == D3D_BF16; }
+  int32_t supportsFormat(int32_t pos, const d3d_tensor_desc* io, int32_t nbIn, int32_t nbOut) const override {
+    if (!io || pos < 0 || pos >= nbIn + nbOut || io[pos].format != D3D_LINEAR) return 0;
+    if (pos == 0) return featureType(io[0].dtype);
+    if (pos == 5) return io[5].dtype == io[0].dtype;  // mm_trt.cu:113
+    return io[pos].dtype == D3D_INT32;
+  }
+
+  // configurePlugin (mm_trt.cu:127-142): weights and bias are rounded to the
+  // feature type exactly as the reference's static_cast<half> does, then
+  // uploaded; the fp32 copy holds the rounded values.
+  int32_t configure(const d3d_tensor_desc* in, int32_t nbIn, const d3d_tensor_desc*, int32_t) override {
+    if (!in || nbIn < 1) return D3D_ERR_BAD_ARG;
+    const int32_t dtype = in[0].dtype;
+    if (!featureType(dtype)) {
+      setError("SPConvMM: feature dtype %d not implemented", dtype);
+      return D3D_ERR_UNSUPPORTED;
+    }
+    std::lock_guard<std::mutex> lock(*devMutex);
+    if (dev->dtype == dtype) return D3D_OK;
+    const size_t nW = static_cast<size_t>(kernelVol) * cin * cout;
+    std::vector<float> w(nW), b(withBias ? cout : 0);
+    std::memcpy(w.data(), blob.data() + weightOffset, nW * 4);
+    if (withBias) std::memcpy(b.data(), blob.data() + weightOffset + nW * 4, static_cast<size_t>(cout) * 4);
+    std::vector<uint16_t> packed;
+    if (dtype == D3D_HALF || dtype == D3D_BF16) {
+      const bool half = dtype == D3D_HALF;
+      auto rnd = [&](float v, uint16_t* bits) {
+        *bits = half ? floatToHalfBits(v) : floatToBf16Bits(v);
+        return half ? halfBitsToFloat(*bits) : bf16BitsToFloat(*bits);
+      };
+      const bool mfma = convUsesMfma(dtype, cin, cout);
+      if (mfma) packed.resize(nW);
+      for (int k = 0; k < kernelVol; ++k)
+        for (int ci = 0; ci < cin; ++ci)
+          for (int co = 0; co < cout; ++co) {
+            const size_t src = (static_cast<size_t>(k) * cin + ci) * cout + co;
+            uint16_t bits;
+            w[src] = rnd(w[src], &bits);
+            if (mfma) packed[(static_cast<size_t>(k) * cout + co) * cin + ci] = bits;  // reduction dim contiguous
+          }
+      for (auto& v : b) {
+        uint16_t bits;
+        v = rnd(v, &bits);
+      }
+    }
+    int32_t rc = dev->f32.upload(w.data(), nW * 4);
+    if (rc != D3D_OK) return rc;
+    if (!packed.empty()) {
+      rc = dev->mfma.upload(packed.data(), nW * 2);
+      if (rc != D3D_OK) return rc;
+    }
+    if (withBias) {
+      rc = dev->bias.upload(b.data(), b.size() * 4);
+      if (rc != D3D_OK) return rc;
+    }
+    dev->dtype = dtype;
+    return D3D_OK;
+  }
+
+  size_t workspaceSize(const d3d_tensor_desc*, int32_t) const override { return 0; }  // mm_trt.cu:143-148
+
+  int32_t enqueue(const d3d_tensor_desc* inDesc, const d3d_tensor_desc* outDesc, const void* const* inputs,
+                  void* const* outputs, void*, size_t, hipStream_t stream) override {
+    if (!inDesc || !outDesc || !inputs || !outputs || !inputs[0] || !inputs[3] || !inputs[4] || !outputs[0]) {
+      setError("SPConvMM: null descriptor or tensor");
+      return D3D_ERR_BAD_ARG;
+    }
+    const int32_t dtype = inDesc[0].dtype;
+    if (!featureType(dtype) || outDesc[0].dtype != dtype) {
+      setError("SPConvMM: feature dtype %d / output dtype %d not implemented", dtype, outDesc[0].dtype);
+      return D3D_ERR_UNSUPPORTED;  // the reference returns -1 here too (mm_trt.cu:204)
+    }
+    if (inDesc[0].nb_dims != 2 || inDesc[0].dims[1] != cin || outDesc[0].nb_dims != 2 ||
+        outDesc[0].dims[1] != cout || inDesc[3].nb_dims != 2 || inDesc[3].dims[0] != 3) {
+      setError("SPConvMM: expected inFeats [*, %d], index [3, *], outFeats [*, %d]", cin, cout);
+      return D3D_ERR_BAD_ARG;
+    }
+    if (dev->dtype != dtype) {  // a plugin enqueued without configurePlugin, or with another dtype
+      int32_t rc = configure(inDesc, 1, nullptr, 0);
+      if (rc != D3D_OK) return rc;
+    }
+    const int64_t rowLen = inDesc[3].dims[1];  // numIndicesMax, mm_trt.cu:169
+    const int64_t outRows = outDesc[0].dims[0];
+    std::shared_ptr<DeviceBuffer> table;
+    int32_t rc = neighbourTable(static_cast<const int32_t*>(inputs[3]), rowLen, static_cast<const int32_t*>(inputs[4]),
+                                inverse, kernelVol, outRows, stream, &table);
+    if (rc != D3D_OK) return rc;
+    lastTable = table;
+    ConvArgs a{};
+    a.dtype = dtype;
+    a.kVol = kernelVol;
+    a.cin = cin;
+    a.cout = cout;
+    a.inRows = inDesc[0].dims[0];
+    a.outRows = outRows;
+    a.in = inputs[0];
+    a.out = outputs[0];
+    a.weightsF32 = static_cast<const float*>(dev->f32.ptr);
+    a.weightsMfma = dev->mfma.ptr;
+    a.bias = withBias ? static_cast<const float*>(dev->bias.ptr) : nullptr;
+    a.nbr = static_cast<const int32_t*>(table->ptr);
+    a.relu = relu ? 1 : 0;
+    return launchConv(a, stream);
+  }
+};
+
+struct OpEntry {
+  const char* name;
+  int nd;  // 0 = SPConvMM
+};
+constexpr OpEntry kOps[] = {{"SPConvIdx1d", 1}, {"SPConvIdx2d", 2}, {"SPConvIdx3d", 3}, {"SPConvIdx4d", 4},
+                            {"SPConvMM", 0}};
+constexpr const char* kVersion = "2.0";
+
+}  // namespace
+}  // namespace d3d
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+using namespace d3d;
+
+#define D3D_GUARD_BEGIN try {
+#define D3D_GUARD_END(ret)                         \
+  }                                                \
+  catch (const std::bad_alloc&) {                  \
+    setError("out of host memory");                \
+    return ret;                                    \
+  }                                                \
+  catch (...) {                                    \
+    setError("unexpected C++ exception");          \
+    return ret;                                    \
+  }
+
+extern "C" {
+
+int32_t d3d_create(const char* name, const char* version, const void* blob, size_t len, d3d_plugin** out) {
+  D3D_GUARD_BEGIN
+  if (!name || !out) {
+    setError("d3d_create: null name or output pointer");
+    return D3D_ERR_BAD_ARG;
+  }
+  *out = nullptr;
+  if (version && std::strcmp(version, kVersion) != 0) {
+    setError("operator %s version %s not registered (have %s)", name, version, kVersion);
+    return D3D_ERR_UNKNOWN_OP;
+  }
+  for (const OpEntry& op : kOps) {
+    if (std::strcmp(name, op.name) != 0) continue;
+    if (op.nd == 0) {
+      MMPlugin* p = nullptr;
+      int32_t rc = MMPlugin::parse(blob, len, &p);
+      *out = p;
+      return rc;
+    }
+    IdxPlugin* p = nullptr;
+    int32_t rc = IdxPlugin::parse(op.nd, blob, len, &p);
+    *out = p;
+    return rc;
+  }
+  setError("operator %s not registered", name);
+  return D3D_ERR_UNKNOWN_OP;
+  D3D_GUARD_END(D3D_ERR_BAD_ARG)
+}
+
+int32_t d3d_clone(const d3d_plugin* p, d3d_plugin** out) {
+  D3D_GUARD_BEGIN
+  if (!p || !out) return D3D_ERR_BAD_ARG;
+  *out = p->clone();
+  return D3D_OK;
+  D3D_GUARD_END(D3D_ERR_BAD_ARG)
+}
+
+void d3d_destroy(d3d_plugin* p) { delete p; }
+
+const char* d3d_plugin_type(const d3d_plugin* p) { return p ? p->type.c_str() : ""; }
+const char* d3d_plugin_version(const d3d_plugin*) { return kVersion; }
+
+size_t d3d_serialize_size(const d3d_plugin* p) { return p ? p->blob.size() : 0; }
+
+int32_t d3d_serialize(const d3d_plugin* p, void* buffer, size_t len) {
+  if (!p || !buffer) return D3D_ERR_BAD_ARG;
+  if (len < p->blob.size()) {
+    setError("serialize: buffer of %zu bytes, %zu needed", len, p->blob.size());
+    return D3D_ERR_BAD_ARG;
+  }
+  std::memcpy(buffer, p->blob.data(), p->blob.size());
+  return D3D_OK;
+}
+
+int32_t d3d_num_outputs(const d3d_plugin* p) { return p ? p->numOutputs() : D3D_ERR_BAD_ARG; }
+
+int32_t d3d_output_dims(const d3d_plugin* p, int32_t output_index, const d3d_tensor_desc* in, int32_t nb_in,
+                        d3d_tensor_desc* out) {
+  D3D_GUARD_BEGIN
+  if (!p) return D3D_ERR_BAD_ARG;
+  return p->outputDims(output_index, in, nb_in, out);
+  D3D_GUARD_END(D3D_ERR_BAD_ARG)
+}
+
+int32_t d3d_output_dtype(const d3d_plugin* p, int32_t output_index, const int32_t* in_dtypes, int32_t nb_in) {
+  if (!p) return D3D_ERR_BAD_ARG;
+  return p->outputDtype(output_index, in_dtypes, nb_in);
+}
+
+int32_t d3d_supports_format(const d3d_plugin* p, int32_t pos, const d3d_tensor_desc* in_out, int32_t nb_in,
+                            int32_t nb_out) {
+  if (!p) return 0;
+  return p->supportsFormat(pos, in_out, nb_in, nb_out);
+}
+
+int32_t d3d_configure(d3d_plugin* p, const d3d_tensor_desc* in, int32_t nb_in, const d3d_tensor_desc* out,
+                      int32_t nb_out) {
+  D3D_GUARD_BEGIN
+  if (!p) return D3D_ERR_BAD_ARG;
+  return p->configure(in, nb_in, out, nb_out);
+  D3D_GUARD_END(D3D_ERR_BAD_ARG)
+}
+
+size_t d3d_workspace_size(const d3d_plugin* p, const d3d_tensor_desc* in, int32_t nb_in, const d3d_tensor_desc*,
+                          int32_t) {
+  if (!p) return 0;
+  return p->workspaceSize(in, nb_in);
+}
+
+int32_t d3d_enqueue(d3d_plugin* p, const d3d_tensor_desc* in_desc, const d3d_tensor_desc* out_desc,
+                    const void* const* inputs, void* const* outputs, void* workspace, size_t workspace_bytes,
+                    void* stream) {
+  D3D_GUARD_BEGIN
+  if (!p) return D3D_ERR_BAD_ARG;
+  return p->enqueue(in_desc, out_desc, inputs, outputs, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+  D3D_GUARD_END(D3D_ERR_BAD_ARG)
+}
+
+const char* d3d_last_error(void) { return lastError(); }
+
+int32_t d3d_num_ops(void) { return static_cast<int32_t>(sizeof(kOps) / sizeof(kOps[0])); }
+const char* d3d_op_name(int32_t i) { return (i >= 0 && i < d3d_num_ops()) ? kOps[i].name : ""; }
+
+void d3d_clear_cache(void) {
+  std::lock_guard<std::mutex> lock(g_cacheMutex);
+  g_cache.clear();
+}
+
+}  // extern "C"

@@ -1,0 +1,160 @@
+"""Sparse-convolution layers wired the way the reference wires its plugins into a
+network: one rulebook per indice key, shared by every convolution that names
+the key (reference: InferSpConvModule, tests/cylinder/test_middle_encoder.py:8-96).
+
+Tensors and workspaces are allocated once at their static capacities; a forward
+pass only enqueues kernels on the current stream (no host synchronisation), so
+it can be captured into a HIP graph.
+"""
+import numpy as np
+import torch
+
+from .plugin import Plugin, TensorDesc
+from .spconv_index import index_blob
+from .spconv_mm import mm_blob
+
+
+def _round_up(v, m):
+    return (v + m - 1) // m * m
+
+
+class SparseTensor:
+    """Features + coordinates + live count + grid, all at static capacity."""
+
+    def __init__(self, feats, coors, num_act, grid, batch=1):
+        self.feats, self.coors, self.num_act, self.grid, self.batch = feats, coors, num_act, list(grid), batch
+
+    @property
+    def capacity(self):
+        return self.coors.shape[0]
+
+
+class Rulebook:
+    """Outputs of one SPConvIdx enqueue, cached under an indice key."""
+
+    def __init__(self, index, num_index, out_coors, num_act_out, out_grid, in_tensor):
+        self.index, self.num_index = index, num_index
+        self.out_coors, self.num_act_out, self.out_grid = out_coors, num_act_out, out_grid
+        self.in_coors, self.num_act_in, self.in_grid = in_tensor.coors, in_tensor.num_act, in_tensor.grid
+
+
+class SparseConvLayer:
+    """One convolution: an SPConvMM plugin plus (for the first user of a key) an SPConvIdx plugin."""
+
+    def __init__(self, spec, weight, bias, max_num_act_out, dtype=torch.float16, device="cuda"):
+        self.spec = spec
+        self.max_num_act_out = int(max_num_act_out)
+        self.dtype = dtype
+        self.device = device
+        nd = len(spec["ksize"])
+        self.idx_plugin = Plugin("SPConvIdx%dd" % nd, index_blob(
+            spec["ksize"], spec["stride"], spec["padding"], spec["dilation"], (0,) * nd, self.max_num_act_out,
+            spec["subm"], spec.get("transpose", False)))
+        self.mm_plugin = Plugin("SPConvMM", mm_blob(
+            spec["ksize"], spec["cin"], spec["cout"], self.max_num_act_out, spec["subm"], spec.get("inverse", False),
+            weight, bias, relu=spec.get("relu", False)))
+        self._idx_state = None
+        self._mm_state = None
+
+    # -- rulebook ---------------------------------------------------------------
+    def build_rulebook(self, x):
+        nd = len(self.spec["ksize"])
+        if self._idx_state is None or self._idx_state["cap"] != x.capacity:
+            in_descs = [TensorDesc.of_tensor(x.coors), TensorDesc.of_tensor(x.num_act),
+                        TensorDesc.of((x.batch, 0) + tuple(x.grid), torch.int32)]
+            out_descs = self.idx_plugin.output_descs(in_descs)
+            outs = [torch.empty(d.shape(), dtype=torch.int32, device=self.device) if 0 not in d.shape() else None
+                    for d in out_descs]
+            ws = torch.empty(max(1, self.idx_plugin.workspace_size(in_descs, out_descs)), dtype=torch.uint8,
+                             device=self.device)
+            self._idx_state = dict(cap=x.capacity, in_descs=in_descs, out_descs=out_descs, outs=outs, ws=ws)
+        st = self._idx_state
+        self.idx_plugin.enqueue(st["in_descs"], st["out_descs"], [x.coors, x.num_act, None], st["outs"], st["ws"])
+        outs = st["outs"]
+        if self.spec["subm"]:  # SubM: outputs sit on the input voxels (test_middle_encoder.py:68-69)
+            return Rulebook(outs[0], outs[1], x.coors, x.num_act, x.grid, x)
+        out_grid = list(st["out_descs"][4].shape()[2:])
+        return Rulebook(outs[0], outs[1], outs[2], outs[3], out_grid, x)
+
+    # -- convolution ------------------------------------------------------------
+    def forward(self, x, rulebooks):
+        key = self.spec["key"]
+        rb = rulebooks.get(key)
+        if rb is None:
+            rb = rulebooks[key] = self.build_rulebook(x)
+        feats = x.feats
+        if self._mm_state is None or self._mm_state["in_rows"] != feats.shape[0]:
+            in_descs = [TensorDesc.of_tensor(t) for t in (feats, rb.num_act_in, rb.num_act_out, rb.index, rb.num_index)]
+            out_descs = self.mm_plugin.output_descs(in_descs)
+            self.mm_plugin.configure(in_descs, out_descs)
+            out = torch.empty(out_descs[0].shape(), dtype=self.dtype, device=self.device)
+            self._mm_state = dict(in_rows=feats.shape[0], in_descs=in_descs, out_descs=out_descs, out=out)
+        st = self._mm_state
+        self.mm_plugin.enqueue(st["in_descs"], st["out_descs"],
+                               [feats, rb.num_act_in, rb.num_act_out, rb.index, rb.num_index], [st["out"]])
+        return SparseTensor(st["out"], rb.out_coors, rb.num_act_out, rb.out_grid, x.batch)
+
+
+class SparseBackbone:
+    """A chain (or small DAG, via ``src``) of SparseConvLayers sharing rulebooks by indice key."""
+
+    def __init__(self, layers, weights, capacities, dtype=torch.float16, device="cuda"):
+        self.specs = layers
+        self.layers = [SparseConvLayer(s, w, b, cap, dtype=dtype, device=device)
+                       for s, (w, b), cap in zip(layers, weights, capacities)]
+
+    def forward(self, x):
+        rulebooks = {}
+        outs = {"input": x}
+        cur = x
+        for spec, lyr in zip(self.specs, self.layers):
+            src = spec.get("src")
+            if src is None:
+                inp = cur
+            elif "+" in src:
+                a, b = (outs[s] for s in src.split("+"))
+                inp = SparseTensor(a.feats + b.feats, a.coors, a.num_act, a.grid, a.batch)
+            else:
+                inp = outs[src]
+            cur = lyr.forward(inp, rulebooks)
+            outs[spec["name"]] = cur
+        self.rulebooks = rulebooks
+        self.outputs = outs
+        return cur
+
+
+def plan_capacities(layers, n_in, counts=None):
+    """Static row capacity (maxNumActOut) of every layer's output.
+
+    SubM layers keep the capacity of their input.  A strided layer's capacity is
+    the measured output count rounded up to 1024 when ``counts[name]`` is given,
+    else the safe bound 8x the input capacity.
+    """
+    caps = []
+    cap_of = {"input": n_in}
+    cur = n_in
+    for spec in layers:
+        src = spec.get("src")
+        if src is not None:
+            cur = cap_of[src.split("+")[0]]
+        if spec["subm"]:
+            cap = cur
+        elif counts is not None and spec["name"] in counts:
+            cap = _round_up(int(counts[spec["name"]]), 1024)
+        else:
+            cap = 8 * cur
+        caps.append(cap)
+        cap_of[spec["name"]] = cap
+        cur = cap
+    return caps
+
+
+def make_input(coords, feats, grid, dtype=torch.float16, device="cuda", capacity=None, batch=1):
+    n = len(coords)
+    capacity = capacity or n
+    c = torch.zeros((capacity, coords.shape[1]), dtype=torch.int32, device=device)
+    c[:n] = torch.from_numpy(np.ascontiguousarray(coords)).to(device)
+    f = torch.zeros((capacity, feats.shape[1]), dtype=dtype, device=device)
+    f[:n] = torch.from_numpy(np.ascontiguousarray(feats)).to(device=device, dtype=dtype)
+    num = torch.tensor([n], dtype=torch.int32, device=device)
+    return SparseTensor(f, c, num, grid, batch)

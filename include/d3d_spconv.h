@@ -1,0 +1,137 @@
+/* C ABI of the MI355X sparse-convolution engine.
+ *
+ * The library exposes the two operators of deploy3d's sparse-convolution path
+ * as opaque plugin objects with the life cycle TensorRT drives on the
+ * reference's IPluginV2DynamicExt classes: deserialize -> clone -> configure
+ * -> workspace size -> enqueue (stream-ordered) -> destroy.  Every function is
+ * noexcept, takes plain pointers and sizes, and returns an int32 status.
+ *
+ * Operator names, version and the packed attribute blobs are the reference's:
+ *   "SPConvIdx1d" .. "SPConvIdx4d", version "2.0"   (trt/spconv/index_trt.cu:20-50, :287-290)
+ *   "SPConvMM",                     version "2.0"   (trt/spconv/mm_trt.cu:22-37, :239)
+ */
+#ifndef D3D_SPCONV_H_
+#define D3D_SPCONV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  0 and -1 are the reference's enqueue() results
+ * (trt/spconv/mm_trt.cu:204); the others replace its print-and-continue. */
+enum {
+  D3D_OK = 0,
+  D3D_ERR_UNSUPPORTED = -1, /* dtype / format / alignment not implemented */
+  D3D_ERR_BAD_BLOB = -2,    /* attribute blob too short or inconsistent */
+  D3D_ERR_BAD_ARG = -3,     /* null pointer, wrong tensor count, wrong dims */
+  D3D_ERR_UNKNOWN_OP = -4,  /* (name, version) not registered */
+  D3D_ERR_WORKSPACE = -5,   /* caller's workspace smaller than d3d_workspace_size() */
+  D3D_ERR_DEVICE = -6       /* a HIP runtime call failed; see d3d_last_error() */
+};
+
+/* Element types; the first five values are nvinfer1::DataType's. */
+enum { D3D_FLOAT = 0, D3D_HALF = 1, D3D_INT8 = 2, D3D_INT32 = 3, D3D_BOOL = 4, D3D_BF16 = 7 };
+
+/* Tensor formats: only row-major linear (nvinfer1::TensorFormat::kLINEAR = 0). */
+enum { D3D_LINEAR = 0 };
+
+#define D3D_MAX_DIMS 8
+
+/* Plain counterpart of nvinfer1::PluginTensorDesc. */
+typedef struct d3d_tensor_desc {
+  int32_t dtype;
+  int32_t format;
+  int32_t nb_dims;
+  int32_t dims[D3D_MAX_DIMS];
+} d3d_tensor_desc;
+
+typedef struct d3d_plugin d3d_plugin;
+
+/* IPluginCreator::deserializePlugin (trt/spconv/index_trt.cu:270-275,
+ * trt/spconv/mm_trt.cu:222-227): the only constructor.  The blob is
+ *   SPConvIdx{N}d: int32 kernelSize[N], stride[N], padding[N], dilation[N],
+ *                  outPadding[N]; int32 maxNumActOut; u8 subM; u8 transpose
+ *                  (packed; trt/spconv/index_trt.cu:39-50)
+ *   SPConvMM:      int32 kernelVol, inChannels, outChannels, maxNumActOut;
+ *                  u8 subM(ignored), inverse, withBias; fp32 W[kVol*Cin*Cout];
+ *                  fp32 bias[Cout] iff withBias  (trt/spconv/mm_trt.cu:27-37, :61-68)
+ *                  optionally followed by a 20-byte extension record
+ *                  {u32 magic 'D3DX'; u32 version 1; u32 flags (bit0 fused ReLU);
+ *                   f32 actScaleIn; f32 actScaleOut} that the reference's parser
+ *                  skips as trailing floats. */
+int32_t d3d_create(const char* name, const char* version, const void* blob, size_t len, d3d_plugin** out);
+
+/* IPluginV2DynamicExt::clone (index_trt.cu:75-79, mm_trt.cu:75-79): clones share device weights. */
+int32_t d3d_clone(const d3d_plugin* p, d3d_plugin** out);
+
+/* destroy() (index_trt.cu:82, mm_trt.cu:82). */
+void d3d_destroy(d3d_plugin* p);
+
+/* getPluginType / getPluginVersion / getPluginNamespace (index_trt.cu:165-168). */
+const char* d3d_plugin_type(const d3d_plugin* p);
+const char* d3d_plugin_version(const d3d_plugin* p);
+
+/* getSerializationSize / serialize (index_trt.cu:70-74, mm_trt.cu:69-74): byte-exact round trip. */
+size_t d3d_serialize_size(const d3d_plugin* p);
+int32_t d3d_serialize(const d3d_plugin* p, void* buffer, size_t len);
+
+/* getNbOutputs (index_trt.cu:98-101: 2 for SubM, 5 otherwise; mm_trt.cu:97). */
+int32_t d3d_num_outputs(const d3d_plugin* p);
+
+/* getOutputDimensions (index_trt.cu:102-151, mm_trt.cu:98-103).  `in` holds the
+ * operator's input descriptors; only their dims are read. */
+int32_t d3d_output_dims(const d3d_plugin* p, int32_t output_index, const d3d_tensor_desc* in, int32_t nb_in,
+                        d3d_tensor_desc* out);
+
+/* getOutputDataType (index_trt.cu:153-155: int32; mm_trt.cu:104-106: type of input 0). */
+int32_t d3d_output_dtype(const d3d_plugin* p, int32_t output_index, const int32_t* in_dtypes, int32_t nb_in);
+
+/* supportsFormatCombination (index_trt.cu:156-161, mm_trt.cu:107-117).  Returns 1 or 0.
+ * Beyond the reference's fp16, SPConvMM also accepts fp32, bf16 and int8 features. */
+int32_t d3d_supports_format(const d3d_plugin* p, int32_t pos, const d3d_tensor_desc* in_out, int32_t nb_in,
+                            int32_t nb_out);
+
+/* configurePlugin (mm_trt.cu:127-142): converts the fp32 weights of the blob to
+ * the feature dtype of in[0] and uploads them (synchronous, default stream). */
+int32_t d3d_configure(d3d_plugin* p, const d3d_tensor_desc* in, int32_t nb_in, const d3d_tensor_desc* out,
+                      int32_t nb_out);
+
+/* getWorkspaceSize (index_trt.cu:178-187, mm_trt.cu:143-148), from capacities only. */
+size_t d3d_workspace_size(const d3d_plugin* p, const d3d_tensor_desc* in, int32_t nb_in, const d3d_tensor_desc* out,
+                          int32_t nb_out);
+
+/* enqueue (index_trt.cu:188-248, mm_trt.cu:149-205).  `stream` is a hipStream_t.
+ * Stream-ordered, no host synchronisation: live counts are read on the device.
+ *
+ * SPConvIdx{N}d  inputs : 0 inCoors int32 [cap, N+1] (b, spatial...), 1 numActIn int32 [1],
+ *                         2 inSpatialShape (dims [B, 0, spatial...] only; pointer unused)
+ *                outputs: 0 index int32 [3, kVol*(cap+128)], 1 numIndex int32 [1],
+ *                         (non-SubM) 2 outCoors int32 [maxNumActOut, N+1], 3 numActOut int32 [1],
+ *                         4 outSpatialShape (dims only)
+ * SPConvMM       inputs : 0 inFeats [capIn, Cin], 1 numActIn [1], 2 numActOut [1],
+ *                         3 index int32 [3, L], 4 numIndex int32 [1]
+ *                outputs: 0 outFeats [maxNumActOut, Cout], dtype of input 0 */
+int32_t d3d_enqueue(d3d_plugin* p, const d3d_tensor_desc* in_desc, const d3d_tensor_desc* out_desc,
+                    const void* const* inputs, void* const* outputs, void* workspace, size_t workspace_bytes,
+                    void* stream);
+
+/* Text of the last error on the calling thread ("" if none).  Replaces the
+ * reference's std::cout reporting (trt/include/common/macros.h:14-34). */
+const char* d3d_last_error(void);
+
+/* Library-wide queries used by loaders: number of registered operators and their names. */
+int32_t d3d_num_ops(void);
+const char* d3d_op_name(int32_t i);
+
+/* Frees every cached neighbour table (the derived, output-major form of an
+ * index tensor that convolutions sharing one indice key reuse).  No reference
+ * counterpart: the reference keeps no derived state between enqueues. */
+void d3d_clear_cache(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* D3D_SPCONV_H_ */

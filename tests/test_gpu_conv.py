@@ -1,0 +1,136 @@
+"""GPU convolution parity: SPConvMM through the C ABI vs the CPU oracle
+(out = bias; for tap: out[scatter] += in[gather] @ W[tap], fp64 accumulation
+on operands rounded to the storage type).
+
+Tolerances (stated by the task): fp32 within 1e-4 relative (|err| <= 1e-4 * (|ref| + rms(ref)));
+fp16 within 2e-2 * rms(ref) absolute; bf16 (an extension) within 8 * 2e-2 * rms(ref), its ulp being 8x fp16's.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import gpu_rulebook, random_cloud
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+TORCH_DTYPE = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
+
+
+def round_to(a, dtype):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(TORCH_DTYPE[dtype]).float().numpy()
+
+
+def check_close(got, ref, dtype):
+    rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2))) + 1e-30
+    err = np.abs(got.astype(np.float64) - ref)
+    if dtype == "float32":
+        bound = 1e-4 * (np.abs(ref) + rms)
+        assert (err <= bound).all(), "fp32: max err %g (rms %g)" % (err.max(), rms)
+    else:
+        tol = 2e-2 * rms * (8 if dtype == "bfloat16" else 1)
+        assert err.max() <= tol, "%s: max err %g > %g (rms %g)" % (dtype, err.max(), tol, rms)
+
+
+def run_case(n, grid, ksize, stride, padding, cin, cout, dtype, subm, with_bias=True, relu=False, inverse=False,
+             seed=0, cap_extra=0):
+    from deploy3d_amd import spconv_mm
+    rng = np.random.default_rng(seed + n + cin * 7 + cout)
+    coords = random_cloud(rng, n, grid, 1)
+    n = len(coords)
+    kvol = int(np.prod(ksize))
+    dil = (1,) * len(ksize)
+    max_out = n if subm else n * 8
+    rb = gpu_rulebook(coords, n, grid, 1, ksize, stride, padding, dil, max_out, subm, cap=n + cap_extra)
+    n_out = n if subm else rb["num_act_out"]
+    in_rows, out_rows = (n + cap_extra, max_out) if not inverse else (max_out, n + cap_extra)
+    feats = round_to(rng.standard_normal((in_rows, cin)), dtype)
+    w = round_to(rng.standard_normal((kvol, cin, cout)) / np.sqrt(kvol * cin), dtype)
+    b = round_to(rng.standard_normal(cout), dtype) if with_bias else None
+    if inverse:
+        cin_, cout_ = cin, cout
+    ref = oracle.conv(feats, w, b, rb["index"], rb["num_index"], out_rows, inverse=inverse, acc="f64")
+    if relu:
+        ref = np.maximum(ref, 0.0)
+    idx_dev, num_index_dev = rb["dev"][0], rb["dev"][1]
+    num_in = rb["num_act_in"]
+    num_out = num_in if subm else rb["dev"][3]
+    if inverse:
+        num_in, num_out = num_out, num_in
+    x = torch.from_numpy(feats).to(device="cuda", dtype=TORCH_DTYPE[dtype])
+    y = spconv_mm(x, num_in, num_out, idx_dev, num_index_dev, ksize, cin, cout, out_rows, subm, inverse, w, b,
+                  relu=relu)
+    torch.cuda.synchronize()
+    got = y.float().cpu().numpy()
+    live = n if (subm or inverse) else n_out
+    check_close(got[:live], ref[:live], dtype)
+    # rows beyond the live outputs hold the (activated) bias, as after the reference's biasInit (trt/spconv/mm.h:51-56)
+    if out_rows > live:
+        tail = np.zeros(cout) if b is None else b.astype(np.float64)
+        if relu:
+            tail = np.maximum(tail, 0)
+        np.testing.assert_allclose(got[live:], np.broadcast_to(round_to(tail, dtype), got[live:].shape), rtol=0, atol=0)
+    return got, ref
+
+
+@pytest.mark.parametrize("cin,cout", [(16, 16), (16, 32), (32, 32), (32, 64), (64, 64), (64, 128), (128, 128),
+                                      (128, 16), (16, 128)])
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_mfma_subm(engine, cin, cout, dtype):
+    run_case(3000, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, dtype, True, relu=(cin == 32))
+
+
+@pytest.mark.parametrize("cin,cout", [(16, 32), (32, 64), (64, 128), (128, 128)])
+def test_mfma_strided(engine, cin, cout):
+    run_case(3000, (10, 36, 30), (3, 3, 3), (2, 2, 2), (1, 1, 1), cin, cout, "float16", False, relu=True)
+
+
+@pytest.mark.parametrize("cin,cout,dtype", [(5, 16, "float16"), (16, 16, "float32"), (3, 7, "float32"),
+                                            (32, 64, "float32"), (40, 24, "float16"), (70, 130, "float32"),
+                                            (5, 16, "bfloat16"), (1, 1, "float32")])
+def test_narrow_subm(engine, cin, cout, dtype):
+    run_case(2500, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, dtype, True, relu=(cout == 16))
+
+
+def test_narrow_strided_fp32(engine):
+    run_case(2500, (10, 36, 30), (3, 3, 3), (2, 2, 2), (1, 1, 1), 16, 16, "float32", False)
+
+
+@pytest.mark.parametrize("ksize,padding", [((3, 1, 3), (1, 0, 1)), ((1, 3, 3), (0, 1, 1)), ((1, 1, 1), (0, 0, 0)),
+                                           ((5, 5, 5), (2, 2, 2))])
+def test_kernel_shapes(engine, ksize, padding):
+    run_case(2500, (10, 36, 30), ksize, (1, 1, 1), padding, 32, 64, "float16", True)
+
+
+def test_no_bias_no_relu(engine):
+    run_case(2500, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), 32, 32, "float16", True, with_bias=False)
+
+
+@pytest.mark.parametrize("subm", [True, False])
+@pytest.mark.parametrize("dtype", ["float16", "float32"])
+def test_inverse(engine, subm, dtype):
+    """inverse swaps the gather and scatter rows of the same rulebook (trt/spconv/mm_trt.cu:174-177)."""
+    stride = (1, 1, 1) if subm else (2, 2, 2)
+    run_case(2500, (10, 36, 30), (3, 3, 3), stride, (1, 1, 1), 32, 16, dtype, subm, inverse=True)
+
+
+def test_capacity_rows_beyond_live(engine):
+    run_case(2500, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), 32, 32, "float16", True, cap_extra=777)
+
+
+def test_bit_reproducible(engine):
+    a, _ = run_case(3000, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), 64, 64, "float16", True)
+    b, _ = run_case(3000, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), 64, 64, "float16", True)
+    np.testing.assert_array_equal(a, b)
+
+
+def test_unsupported_dtype_returns_minus_one(engine):
+    """The reference returns -1 from enqueue for a dtype it does not implement (trt/spconv/mm_trt.cu:204)."""
+    from deploy3d_amd import EngineError, spconv_mm
+    x = torch.zeros((128, 16), dtype=torch.int32, device="cuda")
+    idx = torch.full((3, 27 * 256), -1, dtype=torch.int32, device="cuda")
+    one = torch.zeros(1, dtype=torch.int32, device="cuda")
+    with pytest.raises((EngineError, KeyError)) as e:
+        spconv_mm(x, one, one, idx, one, (3, 3, 3), 16, 16, 128, True, False, np.zeros(27 * 16 * 16, np.float32))
+    if isinstance(e.value, EngineError):
+        assert e.value.status == -1

@@ -1,0 +1,160 @@
+"""GPU rulebook parity: SPConvIdx{N}d through the C ABI vs the CPU oracle.
+
+Bar: output coordinates and index pairs bit-exact after the canonical sort; for
+SubM (where output ids are input rows) the whole index tensor is compared
+bit for bit, padding included.
+"""
+import numpy as np
+import pytest
+
+from helpers import check_index_structure, gpu_rulebook, random_cloud
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+SUBM_CASES = [
+    # (n, grid, batch, ksize, padding, dilation)
+    (500, (9, 20, 18), 2, (3, 3, 3), (1, 1, 1), (1, 1, 1)),
+    (3000, (12, 40, 33), 1, (3, 3, 3), (1, 1, 1), (1, 1, 1)),
+    (2000, (12, 40, 33), 1, (3, 1, 3), (1, 0, 1), (1, 1, 1)),
+    (2000, (12, 40, 33), 1, (1, 3, 3), (0, 1, 1), (1, 1, 1)),
+    (2000, (16, 30, 30), 1, (3, 3, 3), (2, 2, 2), (2, 2, 2)),
+    (1500, (10, 25, 25), 1, (5, 3, 1), (2, 1, 0), (1, 1, 1)),
+    (700, (64, 64), 1, (3, 3), (1, 1), (1, 1)),
+    (300, (500,), 2, (5,), (2,), (1,)),
+    (1000, (6, 8, 10, 12), 1, (3, 3, 3, 3), (1, 1, 1, 1), (1, 1, 1, 1)),
+    (20000, (41, 160, 140), 1, (3, 3, 3), (1, 1, 1), (1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", SUBM_CASES, ids=lambda c: "n%d_k%s" % (c[0], "x".join(map(str, c[3]))))
+def test_subm_matches_oracle_bit_exact(engine, case):
+    n, grid, batch, ksize, padding, dilation = case
+    rng = np.random.default_rng(1000 + n)
+    coords = random_cloud(rng, n, grid, batch)
+    n = len(coords)
+    stride = (1,) * len(ksize)
+    ref = oracle.rulebook(coords, n, (batch,) + grid, ksize, stride, padding, dilation, n, True)
+    got = gpu_rulebook(coords, n, grid, batch, ksize, stride, padding, dilation, n, True)
+    assert got["num_index"] == ref["num_index"]
+    np.testing.assert_array_equal(got["index"], ref["index"])
+    check_index_structure(got["index"], got["num_index"], int(np.prod(ksize)), n)
+
+
+CONV_CASES = [
+    # (n, grid, batch, ksize, stride, padding, dilation, transpose)
+    (500, (9, 20, 18), 2, (3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1), False),
+    (3000, (12, 40, 33), 1, (3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1), False),
+    (3000, (12, 40, 33), 1, (3, 3, 3), (2, 2, 2), (0, 1, 1), (1, 1, 1), False),
+    (3000, (12, 40, 33), 1, (3, 1, 1), (2, 1, 1), (0, 0, 0), (1, 1, 1), False),
+    (3000, (12, 40, 33), 1, (3, 3, 3), (2, 2, 1), (1, 1, 1), (1, 1, 1), False),
+    (2000, (12, 40, 33), 1, (2, 2, 2), (2, 2, 2), (0, 0, 0), (1, 1, 1), False),
+    (2000, (12, 40, 33), 1, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), False),
+    (2000, (12, 40, 33), 1, (3, 3, 3), (3, 2, 1), (1, 0, 2), (2, 1, 1), False),
+    (1000, (6, 20, 16), 1, (3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1), True),
+    (1000, (6, 20, 16), 1, (2, 2, 2), (2, 2, 2), (0, 0, 0), (1, 1, 1), True),
+    (700, (64, 64), 1, (3, 3), (2, 2), (1, 1), (1, 1), False),
+    (300, (500,), 2, (3,), (2,), (1,), (1,), False),
+    (800, (6, 8, 10, 12), 1, (3, 3, 3, 3), (2, 2, 2, 2), (1, 1, 1, 1), (1, 1, 1, 1), False),
+    (20000, (41, 160, 140), 1, (3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1), False),
+]
+
+
+def _conv_case(case, max_out=None, cap=None):
+    n, grid, batch, ksize, stride, padding, dilation, transpose = case
+    rng = np.random.default_rng(2000 + n + 7 * int(transpose))
+    coords = random_cloud(rng, n, grid, batch)
+    n = len(coords)
+    out_grid = oracle.out_shape(grid, ksize, stride, padding, dilation, None, transpose)
+    kvol = int(np.prod(ksize))
+    full = max_out is None
+    max_out = n * kvol if full else max_out
+    ref = oracle.rulebook(coords, n, [batch] + out_grid, ksize, stride, padding, dilation, max_out, False, transpose)
+    got = gpu_rulebook(coords, n, grid, batch, ksize, stride, padding, dilation, max_out, False, transpose, cap=cap)
+    return coords, out_grid, ref, got, kvol
+
+
+@pytest.mark.parametrize("case", CONV_CASES,
+                         ids=lambda c: "n%d_k%s_s%s%s" % (c[0], "x".join(map(str, c[3])), "x".join(map(str, c[4])),
+                                                          "_T" if c[7] else ""))
+def test_conv_matches_oracle_canonical(engine, case):
+    coords, out_grid, ref, got, kvol = _conv_case(case)
+    assert got["out_grid"] == out_grid
+    assert got["num_act_out"] == ref["num_act_out"]
+    assert got["num_index"] == ref["num_index"]
+    c_ref, t_ref = oracle.canonical(ref["index"], ref["num_index"], ref["out_coors"], ref["num_act_out"])
+    c_got, t_got = oracle.canonical(got["index"], got["num_index"], got["out_coors"], got["num_act_out"])
+    np.testing.assert_array_equal(c_got, c_ref)
+    np.testing.assert_array_equal(t_got, t_ref)
+    check_index_structure(got["index"], got["num_index"], kvol, len(coords))
+
+
+def test_conv_output_order_is_deterministic(engine):
+    case = CONV_CASES[1]
+    _, _, _, a, _ = _conv_case(case)
+    _, _, _, b, _ = _conv_case(case)
+    np.testing.assert_array_equal(a["index"], b["index"])
+    np.testing.assert_array_equal(a["out_coors"][:a["num_act_out"]], b["out_coors"][:b["num_act_out"]])
+
+
+@pytest.mark.parametrize("max_out", [1, 100, 1000])
+def test_conv_truncation_keeps_a_consistent_subset(engine, max_out):
+    """numActOut = min(total, maxNumActOut); survivors are unique members of the full output set and the
+    pairs are exactly the full rulebook's pairs restricted to them (tests/spconv/test_spconv.py:72-124)."""
+    case = CONV_CASES[1]
+    coords, out_grid, full_ref, _, kvol = _conv_case(case)
+    _, _, _, got, _ = _conv_case(case, max_out=max_out)
+    total = full_ref["num_act_out"]
+    assert got["num_act_out"] == min(total, max_out)
+    full_set = {tuple(c): i for i, c in enumerate(full_ref["out_coors"][:total].tolist())}
+    kept = [tuple(c) for c in got["out_coors"][:got["num_act_out"]].tolist()]
+    assert len(set(kept)) == len(kept) and all(k in full_set for k in kept)
+    # pairs of the full rulebook restricted to survivors, in coordinate terms
+    ni = full_ref["num_index"]
+    g, s, t = full_ref["index"][:, :ni]
+    live = t >= 0
+    ref_pairs = {(int(tt), int(gg), tuple(full_ref["out_coors"][ss])) for gg, ss, tt in
+                 zip(g[live], s[live], t[live]) if tuple(full_ref["out_coors"][ss]) in set(kept)}
+    ni = got["num_index"]
+    g, s, t = got["index"][:, :ni]
+    live = t >= 0
+    got_pairs = {(int(tt), int(gg), tuple(got["out_coors"][ss])) for gg, ss, tt in zip(g[live], s[live], t[live])}
+    assert got_pairs == ref_pairs
+    check_index_structure(got["index"], got["num_index"], kvol, len(coords))
+
+
+def test_capacity_larger_than_live_count(engine):
+    """cap > numActIn: rows beyond the live count are ignored (test_spconv.py:167-168 uses 20000 of 40000)."""
+    case = CONV_CASES[1]
+    coords, out_grid, ref, got, kvol = _conv_case(case, cap=2 * case[0])
+    c_ref, t_ref = oracle.canonical(ref["index"], ref["num_index"], ref["out_coors"], ref["num_act_out"])
+    c_got, t_got = oracle.canonical(got["index"], got["num_index"], got["out_coors"], got["num_act_out"])
+    np.testing.assert_array_equal(c_got, c_ref)
+    np.testing.assert_array_equal(t_got, t_ref)
+    assert got["index"].shape[1] == kvol * (2 * case[0] + 128)
+
+
+def test_empty_input(engine):
+    """numActIn = 0 => numIndex = 0 and numActOut = 0 (trt/spconv/index.cu:271-275, :414-417)."""
+    coords = np.zeros((256, 4), dtype=np.int32)
+    got = gpu_rulebook(coords, 0, (8, 8, 8), 1, (3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1), 100, False)
+    assert got["num_index"] == 0 and got["num_act_out"] == 0
+    got = gpu_rulebook(coords, 0, (8, 8, 8), 1, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 256, True)
+    assert got["num_index"] == 0
+    assert (got["index"] == -1).all()
+
+
+def test_single_voxel_and_full_block(engine):
+    one = np.array([[0, 2, 3, 4]], dtype=np.int32)
+    got = gpu_rulebook(one, 1, (5, 6, 7), 1, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1, True)
+    assert got["num_index"] == 128
+    live = got["index"][2] >= 0
+    assert live.sum() == 1 and got["index"][2][live][0] == 13 and got["index"][0][live][0] == 0
+    # a full dense block: every interior voxel has all 27 neighbours
+    zz, yy, xx = np.meshgrid(np.arange(4), np.arange(5), np.arange(6), indexing="ij")
+    block = np.stack([np.zeros(120, dtype=np.int64), zz.ravel(), yy.ravel(), xx.ravel()], 1).astype(np.int32)
+    got = gpu_rulebook(block, 120, (4, 5, 6), 1, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 120, True)
+    live = got["index"][2] >= 0
+    expected = sum((4 - abs(dz)) * (5 - abs(dy)) * (6 - abs(dx)) for dz in (-1, 0, 1) for dy in (-1, 0, 1)
+                   for dx in (-1, 0, 1))
+    assert live.sum() == expected
