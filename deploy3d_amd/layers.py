@@ -149,6 +149,33 @@ def plan_capacities(layers, n_in, counts=None):
     return caps
 
 
+def measure_output_counts(layers, coords, grid, batch=1, device="cuda"):
+    """Sizing pre-pass (set-up time, synchronises): live output count of every strided layer of a chain,
+    found by running its rulebook at the safe capacity min(8 * inputs, output cells)."""
+    from .spconv_index import spconv_index_nd
+    counts = {}
+    cur = torch.from_numpy(np.ascontiguousarray(coords)).to(device)
+    cur_grid = list(grid)
+    seen = set()
+    for spec in layers:
+        if spec["subm"] or spec["key"] in seen:
+            continue
+        seen.add(spec["key"])
+        n = cur.shape[0]
+        out_grid = [(i + 2 * p - d * (k - 1) - 1) // s + 1 for i, k, s, p, d in
+                    zip(cur_grid, spec["ksize"], spec["stride"], spec["padding"], spec["dilation"])]
+        cap_out = int(min(8 * n, batch * int(np.prod(out_grid))))
+        num = torch.tensor([n], dtype=torch.int32, device=device)
+        shape = torch.empty((batch, 0) + tuple(cur_grid), dtype=torch.int32, device=device)
+        _, _, out_coors, num_out, _ = spconv_index_nd(cur, num, shape, spec["ksize"], spec["stride"], spec["padding"],
+                                                      spec["dilation"], (0,) * len(out_grid), cap_out, False, False)
+        m = int(num_out.item())
+        counts[spec["name"]] = m
+        cur = out_coors[:m].contiguous()
+        cur_grid = out_grid
+    return counts
+
+
 def make_input(coords, feats, grid, dtype=torch.float16, device="cuda", capacity=None, batch=1):
     n = len(coords)
     capacity = capacity or n

@@ -1,0 +1,62 @@
+"""Runs a layer table (deploy3d_amd.synth) through the CPU oracle, mirroring the
+wiring of deploy3d_amd.layers.SparseBackbone: one rulebook per indice key, bias
+and weights rounded to the storage type, fp64 accumulation, one rounding of the
+output to the storage type, ReLU where the layer fuses it.
+"""
+import numpy as np
+import torch
+
+from oracle import oracle
+
+TORCH_DTYPE = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
+
+
+def round_to(a, dtype):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(TORCH_DTYPE[dtype]).float().numpy()
+
+
+def oracle_chain(cfg, threads=1, acc="f64"):
+    """Returns dict name -> dict(feats [n, C] float32 (storage-rounded), coords [n, 4], grid, pairs P)."""
+    dtype = cfg["dtype"]
+    coords = cfg["coords"]
+    outs = {"input": dict(feats=round_to(cfg["feats"], dtype), coords=coords, grid=list(cfg["grid"]))}
+    rulebooks = {}
+    cur = outs["input"]
+    for spec, (w, b) in zip(cfg["layers"], cfg["weights"]):
+        src = spec.get("src")
+        if src is None:
+            x = cur
+        elif "+" in src:
+            a, c = (outs[s] for s in src.split("+"))
+            x = dict(feats=round_to(a["feats"] + c["feats"], dtype), coords=a["coords"], grid=a["grid"])
+        else:
+            x = outs[src]
+        n = len(x["coords"])
+        rb = rulebooks.get(spec["key"])
+        if rb is None:
+            if spec["subm"]:
+                rb = oracle.rulebook(x["coords"], n, [1] + x["grid"], spec["ksize"], spec["stride"], spec["padding"],
+                                     spec["dilation"], n, True)
+                rb.update(out_coors=x["coords"], num_act_out=n, out_grid=x["grid"])
+            else:
+                og = oracle.out_shape(x["grid"], spec["ksize"], spec["stride"], spec["padding"], spec["dilation"])
+                rb = oracle.rulebook(x["coords"], n, [1] + og, spec["ksize"], spec["stride"], spec["padding"],
+                                     spec["dilation"], 8 * n, False)
+                rb["out_coors"] = rb["out_coors"][:rb["num_act_out"]].copy()
+                rb["out_grid"] = og
+            rb["pairs"] = int((rb["index"][2, :rb["num_index"]] >= 0).sum())
+            rulebooks[spec["key"]] = rb
+        n_out = rb["num_act_out"]
+        y = oracle.conv(x["feats"], round_to(w, dtype), round_to(b, dtype), rb["index"], rb["num_index"], n_out,
+                        acc=acc, threads=threads)
+        if spec.get("relu"):
+            y = np.maximum(y, 0)
+        cur = dict(feats=round_to(y, dtype), exact=y, coords=rb["out_coors"], grid=rb["out_grid"],
+                   pairs=rb["pairs"], key=spec["key"])
+        outs[spec["name"]] = cur
+    return outs
+
+
+def sort_rows(coords, feats):
+    order = np.lexsort(np.asarray(coords).T[::-1])
+    return np.asarray(coords)[order], np.asarray(feats)[order]
