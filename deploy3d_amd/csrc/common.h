@@ -47,19 +47,25 @@ struct RbGeom {
 
 // Workspace carve-up of one rulebook build; all offsets in bytes, 256-aligned.
 struct RbWorkspace {
+  bool blockMap;          // dense block map (records) instead of the hash
+  uint32_t nRecords;      // block map: records; nChunks = chunks of 1024 records
+  uint32_t nChunks;
   uint32_t slots;         // hash slots (power of two)
-  uint32_t nBlocks;       // ceil(cap / kRbThreads)
-  size_t table;           // u64 [slots]   key<<32 | value
-  size_t ids;             // u32 [slots]   output row of an occupied slot (strided conv only)
-  size_t staging;         // u32 [kVol, cap] per (tap, input): slot, then output row, or ~0
-  size_t ownPrefix;       // u32 [cap]     (strided conv only)
-  size_t blockOwn;        // u32 [nBlocks] (strided conv only)
-  size_t cnt;             // u32 [kVol, nBlocks] valid pairs per (tap, workgroup)
-  size_t totals;          // u32 [kVol]    valid pairs per tap
+  uint32_t nBlocks;       // input chunks per tap
+  int64_t pitch;          // row pitch of staging, a multiple of the chunk size
+  size_t table;           // hash: u64 [slots] key<<32 | value;  block map: records [nRecords]
+  size_t ids;             // hash: u32 [slots] output row of an occupied slot (strided only);  block map: perm [cap] (SubM)
+  size_t staging;         // u32 [kVol, pitch] per (tap, input): slot, then output row, or ~0
+  size_t ownCnt;          // hash: u32 [kVol, nBlocks] owned outputs per (tap, chunk) (strided only);  block map: chunk totals
+  size_t cnt;             // u32 [kVol, nBlocks] valid pairs per (tap, chunk)
+  size_t totals;          // u32 [2, kVol]  valid pairs per tap; owned outputs per tap
   size_t total;           // bytes
 };
 
-RbWorkspace planRulebookWorkspace(const RbGeom& g, int64_t cap, bool subM);
+// Plan for the structure that will be used given `workspaceBytes` of workspace.
+RbWorkspace planRulebookWorkspace(const RbGeom& g, int64_t cap, bool subM, size_t workspaceBytes);
+// Workspace that is enough for whichever structure gets chosen.  gridKnown = g.shape holds the real output grid.
+size_t rulebookWorkspaceBytes(const RbGeom& g, int64_t cap, bool subM, bool gridKnown);
 
 // Builds one rulebook on `stream`.  coors [cap, nd+1]; numActIn device int32.
 // index [3, rowLen] with rowLen = kVol * (cap + 128).  outCoors / numActOut are
@@ -82,12 +88,14 @@ struct ConvArgs {
   const void* in;
   void* out;
   const float* weightsF32;  // device fp32 [kVol, cin, cout], values already rounded to the storage type
-  const void* weightsMfma;  // device storage-type [kVol, cout, cin] (reduction dim contiguous) or null
+  const void* weightsMfma;  // device storage-type, MFMA fragment-major (see MMPlugin::configure) or null
   const float* bias;      // device fp32 [cout] or null
   const float* requantM;  // int8: per-channel multiplier
   const float* requantB;  // int8: per-channel bias in output quanta
   const int32_t* nbr;     // [kVol, outRows]
+  const void* zeros;      // device, >= 512 zero bytes: the row that absent neighbours gather
   int relu;
+  int tileRows;           // 0 = choose; else rows per workgroup of the MFMA kernel (64, 128 or 256)
 };
 
 int32_t launchConv(const ConvArgs& a, hipStream_t stream);

@@ -22,6 +22,8 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kConvThreads = 256;
 constexpr int kTileRows = 64;
@@ -161,69 +163,107 @@ convNarrow(const T* __restrict__ in, T* __restrict__ out, const float* __restric
 
 // ---------------------------------------------------------------------------
 // MFMA implicit GEMM, fp16 / bf16 storage, fp32 accumulation.
-//   weights: [kVol, COUT, CIN] (reduction dim contiguous), storage type T
-//   tile   : 64 output rows x COUT, 4 wavefronts arranged WAVES_M x WAVES_N
-//   LDS    : gathered rows As[64][CIN+8], weight slice Bs[COUT][CIN+8],
-//            neighbour tile nbT[kVol][64]
+//
+// A wavefront owns 16*MT consecutive output rows and all COUT channels; a
+// workgroup is 4 such wavefronts.  Per tap
+//   * each lane gathers its own operand fragments of the input rows straight
+//     from global memory into registers (16 bytes per load; the four lanes of
+//     a row cover 64 contiguous bytes), zero for rows without this tap, and
+//     the gathers of the next two taps are already in flight while the MFMAs
+//     of the current tap run;
+//   * the weight slice comes from LDS, in the fragment-major order of the
+//     device copy (Wf[tap][kk][n][lane]), so weight reads and row gathers are
+//     tracked by different hardware counters and overlap freely.
+// The product is formed transposed, D^T = W[tap]^T-tile x rows^T, so a lane
+// ends up with 4 consecutive output channels of one row and the epilogue
+// (bias, ReLU, one rounding) stores 8 bytes per lane.
+//
 // Operand layout of v_mfma_f32_16x16x32 (and 16x16x16): lane l supplies row
-// (A) or column (B) l%16 and the (l/16)-th group of 8 (4) consecutive K
-// values; it receives column l%16, rows 4*(l/16)..+3 of the 16x16 result.
+// (first operand) or column (second operand) l%16 and the (l/16)-th group of
+// 8 (4) consecutive K values; it receives column l%16, rows 4*(l/16)..+3.
 // ---------------------------------------------------------------------------
 template <class T> struct Mfma;
 template <> struct Mfma<_Float16> {
-  using Vec8 = half8;
-  __device__ static float4v k32(const Vec8& a, const Vec8& b, const float4v& c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  __device__ static float4v k32(const u32x4& a, const u32x4& b, const float4v& c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0,
+                                                  0);
   }
-  __device__ static float4v k16(const uint2& a, const uint2& b, const float4v& c) {
+  __device__ static float4v k16(const u32x2& a, const u32x2& b, const float4v& c) {
     return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, a), __builtin_bit_cast(half4, b), c, 0, 0,
                                                  0);
   }
 };
 template <> struct Mfma<__bf16> {
-  using Vec8 = bf16x8;
-  __device__ static float4v k32(const Vec8& a, const Vec8& b, const float4v& c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  __device__ static float4v k32(const u32x4& a, const u32x4& b, const float4v& c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                   0, 0);
   }
-  __device__ static float4v k16(const uint2& a, const uint2& b, const float4v& c) {
+  __device__ static float4v k16(const u32x2& a, const u32x2& b, const float4v& c) {
     return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, a), __builtin_bit_cast(short4v, b), c,
                                                      0, 0, 0);
   }
 };
 
-template <class T, int CIN, int COUT, int WAVES_M>
+// Fragment type per K step: 8 elements (16 bytes) when CIN >= 32, else 4.
+template <int CIN> struct Frag { using type = u32x4; };
+template <> struct Frag<16> { using type = u32x2; };
+
+// Weights live in LDS in the same fragment-major order as in global memory:
+// fragment (kk, n) of a tap is 64 consecutive lanes' worth of data, so a
+// wavefront read is one contiguous, conflict-free sweep.
+//
+// RESIDENT = true : the weights of ALL taps fit in LDS.  They are loaded once
+//   in the prologue; after that every wavefront runs alone (its own active-tap
+//   list, no barriers), with the gathers of the next two taps in flight.
+// RESIDENT = false: one tap's weights at a time, double-buffered.  The slice of
+//   tap t+1 travels global -> registers -> idle LDS buffer while tap t
+//   multiplies; one barrier per tap.  Loads are issued oldest-needed-first, because the
+//   vector-memory counter retires in order: waiting for a weight slice must
+//   not drain the younger gathers behind it.
+template <class T, int CIN, int COUT, int MT, bool RESIDENT>
 __global__ void __launch_bounds__(kConvThreads)
-convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wt, const float* __restrict__ bias,
-         const int32_t* __restrict__ nbr, int kVol, int64_t inRows, int64_t outRows, int relu) {
-  constexpr int TM = kTileRows;
-  constexpr int WAVES_N = 4 / WAVES_M;
-  constexpr int WM = TM / WAVES_M, WN = COUT / WAVES_N;
-  constexpr int MT = WM / 16, NT = WN / 16;
-  constexpr int PITCH = CIN + 8;         // elements; 16 bytes of padding staggers LDS banks
-  constexpr int CHUNKS = CIN / 8;        // 16-byte chunks per row
-  static_assert(MT >= 1 && NT >= 1, "tile split");
+convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
+         const int32_t* __restrict__ nbr, const T* __restrict__ zeros, int kVol, int64_t inRows, int64_t outRows,
+         int relu) {
+  constexpr int WM = 16 * MT;            // rows per wavefront
+  constexpr int TM = 4 * WM;             // rows per workgroup
+  constexpr int NT = COUT / 16;          // output-channel tiles
+  constexpr int KSTEP = CIN >= 32 ? 32 : 16;
+  constexpr int KK = CIN / KSTEP;        // K steps per tap
+  constexpr int KG = KSTEP / 4;          // elements per lane per K step
+  constexpr int WFRAGS = KK * NT * 64;   // fragments (lane granules) per tap
+  constexpr int WCHUNKS = CIN * COUT / 8;  // 16-byte chunks per tap
+  constexpr int WPT = (WCHUNKS + kConvThreads - 1) / kConvThreads;
+  using F = typename Frag<CIN>::type;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  T* As = reinterpret_cast<T*>(smem);
-  T* Bs = As + TM * PITCH;
-  int32_t* nbT = reinterpret_cast<int32_t*>(Bs + COUT * PITCH);
-  uint32_t* tapAny = reinterpret_cast<uint32_t*>(nbT + kVol * TM);
+  F* wLds = reinterpret_cast<F*>(smem);  // RESIDENT: [kVol][WFRAGS]; else [2][WFRAGS]
+  int32_t* nbT = reinterpret_cast<int32_t*>(smem + static_cast<size_t>(RESIDENT ? kVol : 2) * CIN * COUT * sizeof(T));
+  int32_t* tapList = nbT + kVol * TM;    // (!RESIDENT) active taps of the tile, then their count
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int waveM = wave % WAVES_M, waveN = wave / WAVES_M;
+  const int r16 = lane & 15, kgrp = lane >> 4;
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * TM;
+  const int32_t* nb = nbT + wave * WM;   // this wavefront's columns of the [kVol][TM] neighbour tile
 
-  // neighbour tile + which taps occur in it
-  for (int t = tid; t < kVol; t += kConvThreads) tapAny[t] = 0;
-  __syncthreads();
+  // neighbour tile
+  if (!RESIDENT)
+    for (int t = tid; t <= kVol; t += kConvThreads) tapList[t] = 0;
+  if (RESIDENT) {  // all weights, once
+    const u32x4* src = reinterpret_cast<const u32x4*>(wf);
+    u32x4* dst = reinterpret_cast<u32x4*>(wLds);
+    for (int e = tid; e < kVol * WCHUNKS; e += kConvThreads) dst[e] = src[e];
+  } else {
+    __syncthreads();
+  }
   for (int e = tid; e < kVol * TM; e += kConvThreads) {
     const int tap = e / TM, r = e % TM;
     const int64_t row = row0 + r;
     int32_t src = row < outRows ? nbr[static_cast<int64_t>(tap) * outRows + row] : -1;
     if (src >= inRows) src = -1;
     nbT[e] = src;
-    if (src >= 0) tapAny[tap] = 1;
+    if (!RESIDENT && src >= 0) tapList[tap] = 1;
   }
   __syncthreads();
 
@@ -233,91 +273,220 @@ convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wt
 #pragma unroll
     for (int n = 0; n < NT; ++n) acc[m][n] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  const int arow = lane & 15, kgrp = lane >> 4;
-
-  for (int tap = 0; tap < kVol; ++tap) {
-    if (!tapAny[tap]) continue;  // workgroup-uniform
-    __syncthreads();             // previous tap's MFMA reads are done
-    for (int e = tid; e < TM * CHUNKS; e += kConvThreads) {
-      const int r = e / CHUNKS, c = e % CHUNKS;
-      const int32_t src = nbT[tap * TM + r];
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (src >= 0) v = *reinterpret_cast<const uint4*>(in + static_cast<size_t>(src) * CIN + c * 8);
-      *reinterpret_cast<uint4*>(As + r * PITCH + c * 8) = v;
+  // Rows without this tap read a row of zeros (one cached line for the whole device) instead of branching
+  // or selecting afterwards: nothing touches the gathered registers until the MFMAs that consume them, so
+  // the loads of a tap issue back to back and stay in flight across the MFMAs of the taps before it.
+  auto gatherRows = [&](int tap, F (&dst)[MT][KK]) __attribute__((always_inline)) {
+    int32_t src[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) src[m] = nb[tap * TM + m * 16 + r16];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const T* rowPtr = (src[m] < 0 ? zeros : in + static_cast<size_t>(src[m]) * CIN) + kgrp * KG;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) dst[m][kk] = *reinterpret_cast<const F*>(rowPtr + kk * KSTEP);
     }
-    const T* wk = wt + static_cast<size_t>(tap) * COUT * CIN;
-    for (int e = tid; e < COUT * CHUNKS; e += kConvThreads) {
-      const int r = e / CHUNKS, c = e % CHUNKS;
-      *reinterpret_cast<uint4*>(Bs + r * PITCH + c * 8) = *reinterpret_cast<const uint4*>(wk + r * CIN + c * 8);
-    }
-    __syncthreads();
-    if constexpr (CIN >= 32) {
+  };
+  auto multiply = [&](const F* wTap, const F (&rows)[MT][KK]) __attribute__((always_inline)) {
 #pragma unroll
-      for (int kk = 0; kk < CIN / 32; ++kk) {
-        typename Mfma<T>::Vec8 a[MT];
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-          a[m] = *reinterpret_cast<const typename Mfma<T>::Vec8*>(As + (waveM * WM + m * 16 + arow) * PITCH + kk * 32 +
-                                                                  kgrp * 8);
-#pragma unroll
-        for (int n = 0; n < NT; ++n) {
-          const auto b = *reinterpret_cast<const typename Mfma<T>::Vec8*>(Bs + (waveN * WN + n * 16 + arow) * PITCH +
-                                                                          kk * 32 + kgrp * 8);
-#pragma unroll
-          for (int m = 0; m < MT; ++m) acc[m][n] = Mfma<T>::k32(a[m], b, acc[m][n]);
-        }
-      }
-    } else {
-      uint2 a[MT];
-#pragma unroll
-      for (int m = 0; m < MT; ++m)
-        a[m] = *reinterpret_cast<const uint2*>(As + (waveM * WM + m * 16 + arow) * PITCH + kgrp * 4);
+    for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
       for (int n = 0; n < NT; ++n) {
-        const uint2 b = *reinterpret_cast<const uint2*>(Bs + (waveN * WN + n * 16 + arow) * PITCH + kgrp * 4);
+        const F wfrag = wTap[(kk * NT + n) * 64 + lane];
 #pragma unroll
-        for (int m = 0; m < MT; ++m) acc[m][n] = Mfma<T>::k16(a[m], b, acc[m][n]);
+        for (int m = 0; m < MT; ++m) {
+          if constexpr (CIN >= 32) {
+            acc[m][n] = Mfma<T>::k32(wfrag, rows[m][kk], acc[m][n]);
+          } else {
+            acc[m][n] = Mfma<T>::k16(wfrag, rows[m][kk], acc[m][n]);
+          }
+        }
+      }
+    }
+  };
+
+  F bufA[MT][KK], bufB[MT][KK], bufC[MT][KK];
+
+  if constexpr (RESIDENT) {
+    // taps that occur among this wavefront's rows (wavefront-uniform masks)
+    unsigned long long active[2] = {0ull, 0ull};
+    for (int tap = 0; tap < kVol; ++tap) {
+      bool any = false;
+      for (int r = lane; r < WM; r += 64) any = any || nb[tap * TM + r] >= 0;
+      if (__ballot(any)) active[tap >> 6] |= 1ull << (tap & 63);
+    }
+    auto nextTap = [&]() __attribute__((always_inline)) -> int {
+      if (active[0]) {
+        const int t = __builtin_ctzll(active[0]);
+        active[0] &= active[0] - 1;
+        return t;
+      }
+      if (active[1]) {
+        const int t = __builtin_ctzll(active[1]);
+        active[1] &= active[1] - 1;
+        return 64 + t;
+      }
+      return -1;
+    };
+    // Three register sets: while tap t multiplies, the gathers of t+1 and t+2 are in flight.  The sets
+    // rotate through loop-carried copies, which pins each gather to the iteration that issues it.  Past
+    // the last tap the pipeline re-gathers the last tap (harmless, cached) instead of branching.
+    int tNow = nextTap();
+    if (tNow >= 0) {
+      int last = tNow;
+      int tNext = nextTap();
+      gatherRows(tNow, bufA);
+      gatherRows(tNext >= 0 ? (last = tNext) : last, bufB);
+      while (tNow >= 0) {
+        const int tFuture = nextTap();
+        gatherRows(tFuture >= 0 ? (last = tFuture) : last, bufC);
+        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMAs they are meant to overlap
+        multiply(wLds + static_cast<size_t>(tNow) * WFRAGS, bufA);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) {
+            bufA[m][kk] = bufB[m][kk];
+            bufB[m][kk] = bufC[m][kk];
+          }
+        tNow = tNext;
+        tNext = tFuture;
+      }
+    }
+  } else {
+    if (tid == 0) {  // compact the flags into a list in place (slot n <= t is written after flag t was read)
+      int n = 0;
+      for (int t = 0; t < kVol; ++t)
+        if (tapList[t]) tapList[n++] = t;
+      tapList[kVol] = n;
+    }
+    __syncthreads();
+    const int nActive = tapList[kVol];
+    if (nActive > 0) {
+      // indices past the end of the list are clamped to the last tap: the pipeline then re-requests data it
+      // already has (cache hits) instead of branching around loads, which keeps every load unconditional
+      auto tapAt = [&](int a) __attribute__((always_inline)) { return tapList[a < nActive ? a : nActive - 1]; };
+      auto loadWeights = [&](int a, u32x4 (&dst)[WPT]) __attribute__((always_inline)) {
+        const u32x4* wk = reinterpret_cast<const u32x4*>(wf + static_cast<size_t>(tapAt(a)) * CIN * COUT);
+#pragma unroll
+        for (int q = 0; q < WPT; ++q) {
+          const int e = tid + q * kConvThreads;
+          dst[q] = wk[(WCHUNKS % kConvThreads == 0 || e < WCHUNKS) ? e : 0];
+        }
+      };
+      auto storeWeights = [&](int buf, const u32x4 (&src)[WPT]) __attribute__((always_inline)) {
+        u32x4* dst = reinterpret_cast<u32x4*>(wLds + buf * WFRAGS);
+#pragma unroll
+        for (int q = 0; q < WPT; ++q) {
+          const int e = tid + q * kConvThreads;
+          if (WCHUNKS % kConvThreads == 0 || e < WCHUNKS) dst[e] = src[q];
+        }
+      };
+      {
+        u32x4 wreg[WPT];
+        loadWeights(0, wreg);
+        gatherRows(tapAt(0), bufA);
+        gatherRows(tapAt(1), bufB);
+        storeWeights(0, wreg);
+      }
+      __syncthreads();
+      // One tap per iteration: tap a multiplies while the weights of a+1 and the rows of a+2 are requested.
+      // The weights are requested first, so waiting for them leaves the younger gathers in flight; the row
+      // sets rotate through loop-carried copies, which pins each gather to the iteration that issues it.
+      for (int a = 0; a < nActive; ++a) {
+        u32x4 wreg[WPT];
+        loadWeights(a + 1, wreg);
+        gatherRows(tapAt(a + 2), bufC);
+        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMAs they are meant to overlap
+        multiply(wLds + (a & 1) * WFRAGS, bufA);
+        __builtin_amdgcn_sched_barrier(0);
+        storeWeights((a + 1) & 1, wreg);
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) {
+            bufA[m][kk] = bufB[m][kk];
+            bufB[m][kk] = bufC[m][kk];
+          }
       }
     }
   }
 
-  // epilogue: bias, ReLU, one rounding to the storage type
+  // epilogue: lane holds channels n*16 + 4*kgrp .. +3 of row (m*16 + r16)
 #pragma unroll
-  for (int n = 0; n < NT; ++n) {
-    const int col = waveN * WN + n * 16 + arow;
-    const float bv = bias ? bias[col] : 0.f;
+  for (int m = 0; m < MT; ++m) {
+    const int64_t row = row0 + wave * WM + m * 16 + r16;
+    if (row >= outRows) continue;
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
+    for (int n = 0; n < NT; ++n) {
+      const int col = n * 16 + kgrp * 4;
+      float v[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int64_t row = row0 + waveM * WM + m * 16 + kgrp * 4 + j;
-        if (row >= outRows) continue;
-        float v = acc[m][n][j] + bv;
-        if (relu) v = v > 0.f ? v : 0.f;
-        Elem<T>::store(out + static_cast<size_t>(row) * COUT + col, v);
+        v[j] = acc[m][n][j] + (bias ? bias[col + j] : 0.f);
+        if (relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
       }
+      T packed[4] = {static_cast<T>(v[0]), static_cast<T>(v[1]), static_cast<T>(v[2]), static_cast<T>(v[3])};
+      *reinterpret_cast<u32x2*>(out + static_cast<size_t>(row) * COUT + col) = __builtin_bit_cast(u32x2, packed);
     }
   }
 }
 
-template <class T, int CIN, int COUT>
-int32_t launchMfmaOne(const ConvArgs& a, hipStream_t stream) {
-  constexpr int WAVES_M = COUT >= 64 ? 2 : 4;
-  const size_t lds = static_cast<size_t>(kTileRows + COUT) * (CIN + 8) * sizeof(T) +
-                     static_cast<size_t>(a.kVol) * kTileRows * 4 + static_cast<size_t>(a.kVol) * 4;
-  if (lds > 160 * 1024) {
-    setError("conv: %zu bytes of LDS needed (kVol %d too large for the MFMA kernel)", lds, a.kVol);
+constexpr size_t kLdsLimit = 160 * 1024;
+
+template <class T, int CIN, int COUT, int MT, bool RESIDENT>
+int32_t launchMfmaTile(const ConvArgs& a, hipStream_t stream) {
+  constexpr int TM = 64 * MT;
+  const size_t lds = static_cast<size_t>(RESIDENT ? a.kVol : 2) * CIN * COUT * sizeof(T) +
+                     static_cast<size_t>(a.kVol) * TM * sizeof(int32_t) + (static_cast<size_t>(a.kVol) + 1) * 4;
+  if (lds > kLdsLimit) {
+    setError("conv: kernel volume %d too large for the MFMA kernel", a.kVol);
     return D3D_ERR_UNSUPPORTED;
   }
-  if (lds > 64 * 1024) {  // beyond the default dynamic-LDS limit: raise it for this instantiation
-    D3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&convMfma<T, CIN, COUT, WAVES_M>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+  static size_t granted = 64 * 1024;  // dynamic LDS beyond 64 KiB has to be requested per kernel
+  if (lds > granted) {
+    D3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&convMfma<T, CIN, COUT, MT, RESIDENT>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsLimit)));
+    granted = kLdsLimit;
   }
-  const dim3 grid(static_cast<unsigned>((a.outRows + kTileRows - 1) / kTileRows));
-  hipLaunchKernelGGL((convMfma<T, CIN, COUT, WAVES_M>), grid, dim3(kConvThreads), lds, stream,
+  const dim3 grid(static_cast<unsigned>((a.outRows + TM - 1) / TM));
+  hipLaunchKernelGGL((convMfma<T, CIN, COUT, MT, RESIDENT>), grid, dim3(kConvThreads), lds, stream,
                      static_cast<const T*>(a.in), static_cast<T*>(a.out), static_cast<const T*>(a.weightsMfma), a.bias,
-                     a.nbr, a.kVol, a.inRows, a.outRows, a.relu);
+                     a.nbr, static_cast<const T*>(a.zeros), a.kVol, a.inRows, a.outRows, a.relu);
   return D3D_OK;
+}
+
+// Rows per wavefront (16*MT): more rows amortise the weight fragments over more MFMAs; fewer rows give
+// more workgroups per CU to hide the gather latency and to fill 256 CUs.
+template <class T, int CIN, int COUT>
+int32_t launchMfmaOne(const ConvArgs& a, hipStream_t stream) {
+  const size_t allTaps = static_cast<size_t>(a.kVol) * CIN * COUT * sizeof(T);
+  const bool resident = allTaps <= 56 * 1024 && a.kVol <= 128;
+  int mt = resident ? 2 : 4;
+  if (a.tileRows > 0) {
+    mt = a.tileRows / 64;
+  } else {
+    while (mt > 1 && (a.outRows + 64 * mt - 1) / (64 * mt) < 512) mt >>= 1;
+  }
+  auto ldsFor = [&](int m) {
+    return (resident ? allTaps : 2 * static_cast<size_t>(CIN) * COUT * sizeof(T)) +
+           static_cast<size_t>(a.kVol) * 64 * m * 4 + (static_cast<size_t>(a.kVol) + 1) * 4;
+  };
+  while (mt > 1 && ldsFor(mt) > kLdsLimit) mt >>= 1;
+  if (resident) {
+    switch (mt) {
+      case 4: return launchMfmaTile<T, CIN, COUT, 4, true>(a, stream);
+      case 2: return launchMfmaTile<T, CIN, COUT, 2, true>(a, stream);
+      default: return launchMfmaTile<T, CIN, COUT, 1, true>(a, stream);
+    }
+  }
+  switch (mt) {
+    case 4: return launchMfmaTile<T, CIN, COUT, 4, false>(a, stream);
+    case 2: return launchMfmaTile<T, CIN, COUT, 2, false>(a, stream);
+    default: return launchMfmaTile<T, CIN, COUT, 1, false>(a, stream);
+  }
 }
 
 template <class T, int CIN>
@@ -382,7 +551,7 @@ int32_t launchConv(const ConvArgs& a, hipStream_t stream) {
   if (a.outRows <= 0) return D3D_OK;
   int32_t rc = D3D_ERR_UNSUPPORTED;
   const bool aligned = ((reinterpret_cast<uintptr_t>(a.in) | reinterpret_cast<uintptr_t>(a.out)) & 15) == 0;
-  if (convUsesMfma(a.dtype, a.cin, a.cout) && aligned && a.weightsMfma) {
+  if (convUsesMfma(a.dtype, a.cin, a.cout) && aligned && a.weightsMfma && a.zeros) {
     rc = a.dtype == D3D_HALF ? launchMfma<_Float16>(a, stream) : launchMfma<__bf16>(a, stream);
   } else {
     switch (a.dtype) {

@@ -5,6 +5,7 @@
 // Reference life cycle being mirrored: SPConvIdxPlugin (trt/spconv/index_trt.cu:52-249)
 // and SPConvMMPlugin (trt/spconv/mm_trt.cu:39-206).
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <mutex>
@@ -373,13 +374,23 @@ struct IdxPlugin final : d3d_plugin {
     return g;
   }
 
+  // output grid [B, spatial...] from the descriptor of the spatial-shape input
+  void outputGrid(const d3d_tensor_desc& shape, int32_t* grid) const {
+    grid[0] = shape.dims[0];
+    if (subM) {  // index_trt.cu:218-219: SubM works on the input grid
+      for (int i = 0; i < nd; ++i) grid[1 + i] = shape.dims[2 + i];
+    } else {
+      outSpatial(shape.dims + 2, grid + 1);
+    }
+  }
+
+  // getWorkspaceSize (index_trt.cu:178-187): from the row capacity, and from the grid when the caller passes it
   size_t workspaceSize(const d3d_tensor_desc* in, int32_t nbIn) const override {
     if (!in || nbIn < 1) return 0;
-    int32_t ones[kMaxSpatial + 1] = {1, 1, 1, 1, 1};
-    RbGeom g = geometry(ones);
-    // the grid only caps the strided hash; size for the capacity bound alone
-    for (int i = 0; i <= kMaxSpatial; ++i) g.shape[i] = 1 << 6;
-    return planRulebookWorkspace(g, in[0].dims[0], subM).total;
+    const bool gridKnown = nbIn >= 3 && in[2].nb_dims == nd + 2;
+    int32_t grid[kMaxSpatial + 1] = {1 << 6, 1 << 6, 1 << 6, 1 << 6, 1 << 6};  // only caps the strided hash
+    if (gridKnown) outputGrid(in[2], grid);
+    return rulebookWorkspaceBytes(geometry(grid), in[0].dims[0], subM, gridKnown);
   }
 
   int32_t enqueue(const d3d_tensor_desc* inDesc, const d3d_tensor_desc* outDesc, const void* const* inputs,
@@ -400,11 +411,8 @@ struct IdxPlugin final : d3d_plugin {
     }
     // output grid: the input's for SubM (index_trt.cu:218-219), else derived from it
     int32_t grid[kMaxSpatial + 1];
-    grid[0] = inDesc[2].dims[0];
-    if (subM) {
-      for (int i = 0; i < nd; ++i) grid[1 + i] = inDesc[2].dims[2 + i];
-    } else {
-      outSpatial(inDesc[2].dims + 2, grid + 1);
+    outputGrid(inDesc[2], grid);
+    if (!subM) {
       if (outDesc[2].nb_dims != 2 || outDesc[2].dims[0] != maxNumActOut || outDesc[2].dims[1] != nd + 1) {
         setError("%s: outCoors must be [%d, %d]", type.c_str(), maxNumActOut, nd + 1);
         return D3D_ERR_BAD_ARG;
@@ -420,6 +428,31 @@ struct IdxPlugin final : d3d_plugin {
     return rc;
   }
 };
+
+// One zero-filled device row shared by every convolution: the source of gathers for absent neighbours.
+const void* zeroRow() {
+  static std::mutex m;
+  static DeviceBuffer* buf = nullptr;  // lives until the process ends
+  std::lock_guard<std::mutex> lock(m);
+  if (!buf) {
+    auto* b = new DeviceBuffer();
+    if (b->reserve(1024) != D3D_OK || hipMemset(b->ptr, 0, 1024) != hipSuccess) {
+      delete b;
+      return nullptr;
+    }
+    buf = b;
+  }
+  return buf->ptr;
+}
+
+// Tuning / test hook: D3D_CONV_TILE_ROWS = 64, 128 or 256 pins the rows per
+// workgroup of the MFMA convolution; unset or anything else = heuristic.
+int tileRowsOverride() {
+  const char* e = std::getenv("D3D_CONV_TILE_ROWS");
+  if (!e) return 0;
+  const int v = std::atoi(e);
+  return (v == 64 || v == 128 || v == 256) ? v : 0;
+}
 
 // --- SPConvMM ----------------------------------------------------------------
 // Attribute layout: SPConvMMPluginParam + fp32 payload, trt/spconv/mm_trt.cu:27-37, :61-68.
@@ -539,13 +572,20 @@ struct MMPlugin final : d3d_plugin {
       };
       const bool mfma = convUsesMfma(dtype, cin, cout);
       if (mfma) packed.resize(nW);
+      // fragment-major copy for the MFMA kernel: Wf[tap][kk][n][lane][j] = W[tap][kk*KS + (lane/16)*KG + j][n*16 + lane%16]
+      // with KS = 32 (16 when cin == 16) and KG = KS/4, so one wavefront load fetches one whole operand fragment
+      const int ks = cin >= 32 ? 32 : 16, kg = ks / 4, nt = cout / 16, kkN = cin / ks;
       for (int k = 0; k < kernelVol; ++k)
         for (int ci = 0; ci < cin; ++ci)
           for (int co = 0; co < cout; ++co) {
             const size_t src = (static_cast<size_t>(k) * cin + ci) * cout + co;
             uint16_t bits;
             w[src] = rnd(w[src], &bits);
-            if (mfma) packed[(static_cast<size_t>(k) * cout + co) * cin + ci] = bits;  // reduction dim contiguous
+            if (mfma) {
+              const int kk = ci / ks, within = ci % ks, lane = (within / kg) * 16 + co % 16, j = within % kg;
+              const size_t dst = (((static_cast<size_t>(k) * kkN + kk) * nt + co / 16) * 64 + lane) * kg + j;
+              packed[dst] = bits;
+            }
           }
       for (auto& v : b) {
         uint16_t bits;
@@ -561,6 +601,10 @@ struct MMPlugin final : d3d_plugin {
     if (withBias) {
       rc = dev->bias.upload(b.data(), b.size() * 4);
       if (rc != D3D_OK) return rc;
+    }
+    if (!zeroRow()) {
+      setError("SPConvMM: could not allocate the zero row");
+      return D3D_ERR_DEVICE;
     }
     dev->dtype = dtype;
     return D3D_OK;
@@ -595,6 +639,7 @@ struct MMPlugin final : d3d_plugin {
                                 inverse, kernelVol, outRows, stream, &table);
     if (rc != D3D_OK) return rc;
     lastTable = table;
+    const void* zeros = zeroRow();
     ConvArgs a{};
     a.dtype = dtype;
     a.kVol = kernelVol;
@@ -609,6 +654,8 @@ struct MMPlugin final : d3d_plugin {
     a.bias = withBias ? static_cast<const float*>(dev->bias.ptr) : nullptr;
     a.nbr = static_cast<const int32_t*>(table->ptr);
     a.relu = relu ? 1 : 0;
+    a.zeros = zeros;
+    a.tileRows = tileRowsOverride();
     return launchConv(a, stream);
   }
 };

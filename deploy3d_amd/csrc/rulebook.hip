@@ -11,15 +11,21 @@
 //    the static capacity and every kernel reads the live count on the device;
 //  * the coordinate hash is one 64-bit slot per entry (key<<32 | value) in
 //    HBM, claimed with a single 64-bit CAS, so a probe is one 8-byte load;
-//  * compaction is ballot/popcount inside a wavefront plus per-workgroup tap
-//    counts; each workgroup sums the counts of its predecessors itself, so no
-//    device-wide scan kernels and no full-capacity staging passes are needed;
-//  * strided outputs are numbered by their first contributing (input row, tap)
-//    via atomicMin, which makes the output order deterministic (the reference
-//    numbers them by hash-slot order, which depends on CAS races);
+//  * every pass runs one workgroup per (chunk of 1024 inputs, tap), so all
+//    kVol*N probes or inserts of a pass are independent and in flight together;
+//  * compaction is a prefix inside the workgroup plus per-(tap, chunk) counts;
+//    each workgroup sums the counts of its predecessors itself, so there are
+//    no device-wide scan kernels;
+//  * a strided output belongs to the contributing pair with the smallest
+//    (input row, tap) code (atomicMin) and outputs are numbered in (tap, input
+//    row) order of their owners, which makes the output order deterministic
+//    (the reference numbers them by hash-slot order, which depends on CAS races);
 //  * the strided hash is sized by the real bound on distinct outputs per input
 //    (product over dims of the largest number of stride-compatible taps), not
 //    by 2*kVol*N slots.
+#include <cstdlib>
+#include <cstring>
+
 #include "common.h"
 
 namespace d3d {
@@ -52,7 +58,8 @@ __device__ __forceinline__ uint32_t hashInsertMin(unsigned long long* table, uin
       if (cur == kEmptySlot) return slot;
     }
     if (static_cast<uint32_t>(cur >> 32) == key) {
-      atomicMin(table + slot, packed);
+      // values only ever decrease, so a (possibly stale) smaller value settles it
+      if (packed < cur) atomicMin(table + slot, packed);
       return slot;
     }
     slot = (slot + 1) & mask;
@@ -74,6 +81,11 @@ __device__ __forceinline__ uint32_t hashLookup(const unsigned long long* table, 
 // Loads coordinate row `i` widened to (batch, 4 spatial).
 __device__ __forceinline__ void loadCoord(const int32_t* coors, int nd, int64_t i, int c[5]) {
   const int32_t* row = coors + i * (nd + 1);
+  if (nd == 3 && (reinterpret_cast<uintptr_t>(coors) & 15) == 0) {  // the common case: one 16-byte load
+    const int4 v = *reinterpret_cast<const int4*>(row);
+    c[0] = v.x; c[1] = 0; c[2] = v.y; c[3] = v.z; c[4] = v.w;
+    return;
+  }
   const int pad = kMaxSpatial - nd;
   c[0] = row[0];
 #pragma unroll
@@ -102,40 +114,18 @@ __device__ __forceinline__ bool tapDim(const RbGeom& g, int dim, int in, int i, 
     out = in * g.s[dim] - g.p[dim] + i * g.d[dim];
   } else {
     const int c = in + g.p[dim] - i * g.d[dim];
-    if (c % g.s[dim] != 0) return false;
-    out = c / g.s[dim];
-  }
-  return out >= 0 && out < g.shape[dim + 1];
-}
-
-// Calls f(tap, valid, offset) for the kVol taps of one input voxel in
-// row-major tap order; offset is the linear offset of the output voxel in the
-// output grid and only meaningful when valid.
-template <class F>
-__device__ __forceinline__ void forEachTap(const RbGeom& g, const int c[5], F&& f) {
-  const bool batchOk = c[0] >= 0 && c[0] < g.shape[0];
-  int tap = 0;
-  for (int i0 = 0; i0 < g.k[0]; ++i0) {
-    int o0;
-    const bool ok0 = tapDim(g, 0, c[1], i0, o0) && batchOk;
-    const uint32_t off0 = static_cast<uint32_t>(c[0]) * g.shape[1] + o0;
-    for (int i1 = 0; i1 < g.k[1]; ++i1) {
-      int o1;
-      const bool ok1 = tapDim(g, 1, c[2], i1, o1) && ok0;
-      const uint32_t off1 = off0 * g.shape[2] + o1;
-      for (int i2 = 0; i2 < g.k[2]; ++i2) {
-        int o2;
-        const bool ok2 = tapDim(g, 2, c[3], i2, o2) && ok1;
-        const uint32_t off2 = off1 * g.shape[3] + o2;
-        for (int i3 = 0; i3 < g.k[3]; ++i3) {
-          int o3;
-          const bool ok3 = tapDim(g, 3, c[4], i3, o3) && ok2;
-          f(tap, ok3, off2 * g.shape[4] + o3);
-          ++tap;
-        }
-      }
+    const int st = g.s[dim];  // uniform: the branches below are scalar
+    if (st == 1) {
+      out = c;
+    } else if (st == 2) {  // an arithmetic shift keeps negative even numerators negative, so the range test drops them
+      if (c & 1) return false;
+      out = c >> 1;
+    } else {
+      if (c % st != 0) return false;
+      out = c / st;
     }
   }
+  return out >= 0 && out < g.shape[dim + 1];
 }
 
 __device__ __forceinline__ int liveCount(const int32_t* numActIn, int64_t cap) {
@@ -207,8 +197,50 @@ rbReset(uint4* table16, int64_t nTable16, int32_t* index, int64_t nIndex, uint32
 }
 
 // ---------------------------------------------------------------------------
-// SubM: coordinate -> row map (reference: setSubMHashKernel, index.cu:174-182)
+// All passes below run one workgroup per (input chunk, tap): blockIdx.y is the
+// tap, blockIdx.x a chunk of kRbChunk consecutive inputs, 4 per thread.  Every
+// (tap, input) item is independent, so the probes and inserts of a pass are all
+// in flight together instead of one voxel walking its taps serially.
 // ---------------------------------------------------------------------------
+constexpr int kRbItems = 4;
+constexpr int kRbChunk = kRbThreads * kRbItems;
+
+// Tap index -> per-dim kernel positions (row-major over the kernel dims;
+// reference: kernelOffsetStride, trt/spconv/geometry.h:106-109).
+__device__ __forceinline__ void tapPositions(const RbGeom& g, int tap, int idx[kMaxSpatial]) {
+#pragma unroll
+  for (int dim = kMaxSpatial - 1; dim >= 0; --dim) {
+    idx[dim] = tap % g.k[dim];
+    tap /= g.k[dim];
+  }
+}
+
+// Output voxel of (input coordinate, tap); false if the tap does not land on
+// the output lattice or falls outside the output grid.
+__device__ __forceinline__ bool tapTarget(const RbGeom& g, const int c[5], const int idx[kMaxSpatial], uint32_t* off) {
+  bool ok = c[0] >= 0 && c[0] < g.shape[0];
+  uint32_t o = static_cast<uint32_t>(c[0]);
+#pragma unroll
+  for (int dim = 0; dim < kMaxSpatial; ++dim) {
+    int v = 0;
+    ok = tapDim(g, dim, c[dim + 1], idx[dim], v) && ok;
+    o = o * static_cast<uint32_t>(g.shape[dim + 1]) + static_cast<uint32_t>(v);
+  }
+  *off = o;
+  return ok;
+}
+
+// Publishes the number of flagged items of this workgroup for its tap.
+__device__ __forceinline__ void publishCount(uint32_t mine, uint32_t* scratch, uint32_t* cnt, uint32_t nBlocks,
+                                             uint32_t* totals) {
+  const uint32_t total = blockSum(mine, scratch);
+  if (threadIdx.x == 0) {
+    cnt[static_cast<size_t>(blockIdx.y) * nBlocks + blockIdx.x] = total;
+    if (total) atomicAdd(&totals[blockIdx.y], total);
+  }
+}
+
+// SubM: coordinate -> row map (reference: setSubMHashKernel, index.cu:174-182)
 __global__ void __launch_bounds__(kRbThreads)
 rbSubmInsert(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
              unsigned long long* table, uint32_t mask) {
@@ -221,46 +253,37 @@ rbSubmInsert(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restr
   hashInsertMin(table, mask, coordOffset(g, c), static_cast<uint32_t>(i));
 }
 
-// Shared tail of the probe / resolve kernels: per-tap valid counts of this
-// workgroup, accumulated in LDS by one lane per wavefront.
-__device__ __forceinline__ void countTap(uint32_t* ldsCnt, int tap, bool valid) {
-  const unsigned long long m = __ballot(valid);
-  if ((threadIdx.x & 63) == 0 && m) atomicAdd(&ldsCnt[tap], static_cast<uint32_t>(__popcll(m)));
-}
-
-__device__ __forceinline__ void publishCounts(const uint32_t* ldsCnt, int kVol, uint32_t* cnt, uint32_t nBlocks,
-                                              uint32_t* totals) {
-  __syncthreads();
-  for (int t = threadIdx.x; t < kVol; t += blockDim.x) {
-    const uint32_t v = ldsCnt[t];
-    cnt[static_cast<size_t>(t) * nBlocks + blockIdx.x] = v;
-    if (v) atomicAdd(&totals[t], v);
-  }
-}
-
 // SubM probe (reference: subMGeometryKernel + SubMHashWriter, index.cu:48-84):
 // staging[tap, i] = row of the voxel at (coord_i + p - tap*d), or ~0.
 __global__ void __launch_bounds__(kRbThreads)
 rbSubmProbe(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
-            const unsigned long long* __restrict__ table, uint32_t mask, uint32_t* __restrict__ staging,
+            int64_t pitch, const unsigned long long* __restrict__ table, uint32_t mask, uint32_t* __restrict__ staging,
             uint32_t* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
-  extern __shared__ uint32_t ldsCnt[];
-  for (int t = threadIdx.x; t < g.kVol; t += blockDim.x) ldsCnt[t] = 0;
-  __syncthreads();
+  __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const bool live = i < n;
-  int c[5] = {0, 0, 0, 0, 0};
-  if (live) loadCoord(coors, g.nd, i, c);
-  if (static_cast<int64_t>(blockIdx.x) * blockDim.x < n) {  // workgroup-uniform
-    forEachTap(g, c, [&](int tap, bool ok, uint32_t off) {
-      uint32_t row = kNone;
-      if (live && ok) row = hashLookup(table, mask, off);
-      if (live) staging[static_cast<size_t>(tap) * cap + i] = row;
-      countTap(ldsCnt, tap, row != kNone);
-    });
+  const int tap = blockIdx.y;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
+  uint32_t found = 0;
+  if (static_cast<int64_t>(blockIdx.x) * kRbChunk < n) {  // workgroup-uniform
+    int idx[kMaxSpatial];
+    tapPositions(g, tap, idx);
+    uint32_t row[kRbItems];
+#pragma unroll
+    for (int j = 0; j < kRbItems; ++j) {
+      row[j] = kNone;
+      const int64_t i = first + j;
+      if (i < n) {
+        int c[5];
+        loadCoord(coors, g.nd, i, c);
+        uint32_t off;
+        if (tapTarget(g, c, idx, &off)) row[j] = hashLookup(table, mask, off);
+      }
+      found += row[j] != kNone;
+    }
+    if (first < n) *reinterpret_cast<uint4*>(staging + static_cast<size_t>(tap) * pitch + first) =
+        make_uint4(row[0], row[1], row[2], row[3]);
   }
-  publishCounts(ldsCnt, g.kVol, cnt, nBlocks, totals);
+  publishCount(found, scratch, cnt, nBlocks, totals);
 }
 
 // ---------------------------------------------------------------------------
@@ -270,79 +293,112 @@ rbSubmProbe(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restri
 // smallest value per key surviving; staging[tap, i] = slot.
 __global__ void __launch_bounds__(kRbThreads)
 rbConvInsert(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
-             unsigned long long* table, uint32_t mask, uint32_t* __restrict__ staging) {
+             int64_t pitch, unsigned long long* table, uint32_t mask, uint32_t* __restrict__ staging) {
   const int n = liveCount(numActIn, cap);
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  int c[5];
-  loadCoord(coors, g.nd, i, c);
-  const uint32_t codeBase = static_cast<uint32_t>(i) * static_cast<uint32_t>(g.kVol);
-  forEachTap(g, c, [&](int tap, bool ok, uint32_t off) {
-    uint32_t slot = kNone;
-    if (ok) slot = hashInsertMin(table, mask, off, codeBase + tap);
-    staging[static_cast<size_t>(tap) * cap + i] = slot;
-  });
-}
-
-// Pass 2: a pair owns its output iff its code is the surviving value.  Counts
-// owned outputs per input and scans them inside the workgroup.
-__global__ void __launch_bounds__(kRbThreads)
-rbConvOwner(RbGeom g, const int32_t* __restrict__ numActIn, int64_t cap, const unsigned long long* __restrict__ table,
-            const uint32_t* __restrict__ staging, uint32_t* __restrict__ ownPrefix, uint32_t* __restrict__ blockOwn) {
-  __shared__ uint32_t scratch[kRbThreads / 64];
-  const int n = liveCount(numActIn, cap);
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  uint32_t own = 0;
-  if (i < n) {
-    const uint32_t codeBase = static_cast<uint32_t>(i) * static_cast<uint32_t>(g.kVol);
-    for (int tap = 0; tap < g.kVol; ++tap) {
-      const uint32_t slot = staging[static_cast<size_t>(tap) * cap + i];
-      if (slot != kNone && static_cast<uint32_t>(table[slot]) == codeBase + tap) ++own;
+  const int tap = blockIdx.y;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
+  if (first >= n) return;
+  int idx[kMaxSpatial];
+  tapPositions(g, tap, idx);
+  uint32_t slot[kRbItems];
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j) {
+    slot[j] = kNone;
+    const int64_t i = first + j;
+    if (i < n) {
+      int c[5];
+      loadCoord(coors, g.nd, i, c);
+      uint32_t off;
+      if (tapTarget(g, c, idx, &off))
+        slot[j] = hashInsertMin(table, mask, off, static_cast<uint32_t>(i) * static_cast<uint32_t>(g.kVol) + tap);
     }
   }
-  uint32_t total;
-  const uint32_t prefix = blockExclusiveScan(own, scratch, &total);
-  if (i < n) ownPrefix[i] = prefix;
-  if (threadIdx.x == 0) blockOwn[blockIdx.x] = total;
+  *reinterpret_cast<uint4*>(staging + static_cast<size_t>(tap) * pitch + first) =
+      make_uint4(slot[0], slot[1], slot[2], slot[3]);
 }
 
-// Pass 3: output rows are numbered in (owner input row, tap) order; writes the
+// A pair owns its output iff its code is the value that survived in the slot.
+__device__ __forceinline__ void loadOwned(const RbGeom& g, int n, int tap, int64_t first, int64_t pitch,
+                                          const unsigned long long* __restrict__ table,
+                                          const uint32_t* __restrict__ staging, uint32_t slot[kRbItems],
+                                          unsigned long long entry[kRbItems], bool own[kRbItems]) {
+  uint4 s4 = make_uint4(kNone, kNone, kNone, kNone);
+  if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<size_t>(tap) * pitch + first);
+  slot[0] = s4.x; slot[1] = s4.y; slot[2] = s4.z; slot[3] = s4.w;
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j) {
+    const int64_t i = first + j;
+    own[j] = false;
+    entry[j] = 0;
+    if (i < n && slot[j] != kNone) {
+      entry[j] = table[slot[j]];
+      own[j] = static_cast<uint32_t>(entry[j]) == static_cast<uint32_t>(i) * static_cast<uint32_t>(g.kVol) + tap;
+    }
+  }
+}
+
+// Pass 2: owners per (tap, chunk).
+__global__ void __launch_bounds__(kRbThreads)
+rbConvOwner(RbGeom g, const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch,
+            const unsigned long long* __restrict__ table, const uint32_t* __restrict__ staging,
+            uint32_t* __restrict__ ownCnt, uint32_t nBlocks, uint32_t* ownTotals) {
+  __shared__ uint32_t scratch[kRbThreads / 64];
+  const int n = liveCount(numActIn, cap);
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
+  uint32_t mine = 0;
+  if (static_cast<int64_t>(blockIdx.x) * kRbChunk < n) {
+    uint32_t slot[kRbItems];
+    unsigned long long entry[kRbItems];
+    bool own[kRbItems];
+    loadOwned(g, n, blockIdx.y, first, pitch, table, staging, slot, entry, own);
+#pragma unroll
+    for (int j = 0; j < kRbItems; ++j) mine += own[j];
+  }
+  publishCount(mine, scratch, ownCnt, nBlocks, ownTotals);
+}
+
+// Pass 3: output rows are numbered in (tap, owner input row) order; writes the
 // output coordinates (reference: coorsOutOrganizeKernel, index.cu:104-121) and
 // numActOut = min(total, maxNumActOut).
 __global__ void __launch_bounds__(kRbThreads)
-rbConvAssign(RbGeom g, const int32_t* __restrict__ numActIn, int64_t cap, const unsigned long long* __restrict__ table,
-             const uint32_t* __restrict__ staging, const uint32_t* __restrict__ ownPrefix,
-             const uint32_t* __restrict__ blockOwn, uint32_t nBlocks, uint32_t* __restrict__ ids,
-             int32_t* __restrict__ outCoors, int32_t* numActOut, int32_t maxNumActOut) {
+rbConvAssign(RbGeom g, const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch,
+             const unsigned long long* __restrict__ table, const uint32_t* __restrict__ staging,
+             const uint32_t* __restrict__ ownCnt, uint32_t nBlocks, const uint32_t* __restrict__ ownTotals,
+             uint32_t* __restrict__ ids, int32_t* __restrict__ outCoors, int32_t* numActOut, int32_t maxNumActOut) {
   __shared__ uint32_t scratch[kRbThreads / 64];
-  uint32_t before = 0, all = 0;
-  for (uint32_t b = threadIdx.x; b < nBlocks; b += blockDim.x) {
-    const uint32_t v = blockOwn[b];
-    all += v;
-    if (b < blockIdx.x) before += v;
-  }
-  const uint32_t base = blockSum(before, scratch);
-  if (blockIdx.x == 0) {
-    const uint32_t total = blockSum(all, scratch);
-    if (threadIdx.x == 0)
-      *numActOut = static_cast<int32_t>(total < static_cast<uint32_t>(maxNumActOut) ? total : maxNumActOut);
+  const int tap = blockIdx.y;
+  if (blockIdx.x == 0 && tap == 0 && threadIdx.x == 0) {
+    uint32_t total = 0;
+    for (int t = 0; t < g.kVol; ++t) total += ownTotals[t];
+    *numActOut = static_cast<int32_t>(total < static_cast<uint32_t>(maxNumActOut) ? total : maxNumActOut);
   }
   const int n = liveCount(numActIn, cap);
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  uint32_t next = base + ownPrefix[i];
-  const uint32_t codeBase = static_cast<uint32_t>(i) * static_cast<uint32_t>(g.kVol);
+  if (static_cast<int64_t>(blockIdx.x) * kRbChunk >= n) return;  // workgroup-uniform
+  if (ownCnt[static_cast<size_t>(tap) * nBlocks + blockIdx.x] == 0) return;
+  uint32_t before = 0;
+  for (uint32_t q = threadIdx.x; q < blockIdx.x; q += blockDim.x) before += ownCnt[static_cast<size_t>(tap) * nBlocks + q];
+  uint32_t base = blockSum(before, scratch);
+  for (int t = 0; t < tap; ++t) base += ownTotals[t];
+
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
+  uint32_t slot[kRbItems];
+  unsigned long long entry[kRbItems];
+  bool own[kRbItems];
+  loadOwned(g, n, tap, first, pitch, table, staging, slot, entry, own);
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j) mine += own[j];
+  uint32_t total;
+  uint32_t next = base + blockExclusiveScan(mine, scratch, &total);
   const int cw = g.nd + 1;
   const int pad = kMaxSpatial - g.nd;
-  for (int tap = 0; tap < g.kVol; ++tap) {
-    const uint32_t slot = staging[static_cast<size_t>(tap) * cap + i];
-    if (slot == kNone) continue;
-    const unsigned long long entry = table[slot];
-    if (static_cast<uint32_t>(entry) != codeBase + tap) continue;
-    ids[slot] = next;
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j) {
+    if (!own[j]) continue;
+    ids[slot[j]] = next;
     if (next < static_cast<uint32_t>(maxNumActOut)) {
       // reference: Size::deserialize, trt/include/common/refnd.h:56-64
-      uint32_t off = static_cast<uint32_t>(entry >> 32);
+      uint32_t off = static_cast<uint32_t>(entry[j] >> 32);
       int32_t* row = outCoors + static_cast<size_t>(next) * cw;
 #pragma unroll
       for (int dim = kMaxSpatial; dim >= 1; --dim) {
@@ -358,45 +414,46 @@ rbConvAssign(RbGeom g, const int32_t* __restrict__ numActIn, int64_t cap, const 
 }
 
 // Pass 4: slot -> output row, dropping outputs beyond maxNumActOut
-// (reference: hashOutIndexKernel, index.cu:158-172), plus per-tap counts.
+// (reference: hashOutIndexKernel, index.cu:158-172), plus per-(tap, chunk) counts.
 __global__ void __launch_bounds__(kRbThreads)
-rbConvResolve(RbGeom g, const int32_t* __restrict__ numActIn, int64_t cap, const uint32_t* __restrict__ ids,
+rbConvResolve(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, const uint32_t* __restrict__ ids,
               uint32_t* __restrict__ staging, int32_t maxNumActOut, uint32_t* __restrict__ cnt, uint32_t nBlocks,
               uint32_t* totals) {
-  extern __shared__ uint32_t ldsCnt[];
-  for (int t = threadIdx.x; t < g.kVol; t += blockDim.x) ldsCnt[t] = 0;
-  __syncthreads();
+  __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const bool live = i < n;
-  if (static_cast<int64_t>(blockIdx.x) * blockDim.x < n) {  // workgroup-uniform
-    for (int tap = 0; tap < g.kVol; ++tap) {
+  const int tap = blockIdx.y;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
+  uint32_t found = 0;
+  if (first < n) {
+    uint4* cell = reinterpret_cast<uint4*>(staging + static_cast<size_t>(tap) * pitch + first);
+    const uint4 s4 = *cell;
+    uint32_t v[kRbItems] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+    for (int j = 0; j < kRbItems; ++j) {
       uint32_t row = kNone;
-      if (live) {
-        const uint32_t slot = staging[static_cast<size_t>(tap) * cap + i];
-        if (slot != kNone) {
-          const uint32_t id = ids[slot];
-          if (id < static_cast<uint32_t>(maxNumActOut)) row = id;
-        }
-        staging[static_cast<size_t>(tap) * cap + i] = row;
+      if (first + j < n && v[j] != kNone) {
+        const uint32_t id = ids[v[j]];
+        if (id < static_cast<uint32_t>(maxNumActOut)) row = id;
       }
-      countTap(ldsCnt, tap, row != kNone);
+      v[j] = row;
+      found += row != kNone;
     }
+    *cell = make_uint4(v[0], v[1], v[2], v[3]);
   }
-  publishCounts(ldsCnt, g.kVol, cnt, nBlocks, totals);
+  publishCount(found, scratch, cnt, nBlocks, totals);
 }
 
 // ---------------------------------------------------------------------------
 // Compaction (reference: Valid_Counter scan + outputIndexPadOrganizeKernel +
-// indexOrganizeKernel, index.cu:123-156, :352-366).  Workgroup (b, tap) writes
-// the valid pairs of inputs [256b, 256b+256) of one tap at
-//   segment start of the tap  +  pairs of that tap in earlier workgroups  +  rank.
+// indexOrganizeKernel, index.cu:123-156, :352-366).  Workgroup (chunk, tap)
+// writes the valid pairs of its inputs at
+//   segment start of the tap  +  pairs of that tap in earlier chunks  +  rank.
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(kRbThreads)
-rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int kVol, const uint32_t* __restrict__ staging,
-          const uint32_t* __restrict__ cnt, uint32_t nBlocks, const uint32_t* __restrict__ totals,
-          int32_t* __restrict__ gather, int32_t* __restrict__ scatter, int32_t* __restrict__ tapRow,
-          int32_t* numIndex) {
+rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int kVol,
+          const uint32_t* __restrict__ staging, const uint32_t* __restrict__ cnt, uint32_t nBlocks,
+          const uint32_t* __restrict__ totals, int32_t* __restrict__ gather, int32_t* __restrict__ scatter,
+          int32_t* __restrict__ tapRow, int32_t* numIndex) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int tap = blockIdx.y;
   const uint32_t b = blockIdx.x;
@@ -406,7 +463,7 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int kVol, const uin
     *numIndex = static_cast<int32_t>(end);
   }
   const int n = liveCount(numActIn, cap);
-  if (static_cast<int64_t>(b) * blockDim.x >= n) return;  // workgroup-uniform
+  if (static_cast<int64_t>(b) * kRbChunk >= n) return;           // workgroup-uniform
   if (cnt[static_cast<size_t>(tap) * nBlocks + b] == 0) return;  // workgroup-uniform
 
   uint32_t before = 0;
@@ -414,15 +471,472 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int kVol, const uin
   uint32_t pos = blockSum(before, scratch);
   for (int t = 0; t < tap; ++t) pos += (totals[t] + (kSegment - 1)) & ~static_cast<uint32_t>(kSegment - 1);
 
-  const int64_t i = static_cast<int64_t>(b) * blockDim.x + threadIdx.x;
-  const uint32_t row = i < n ? staging[static_cast<size_t>(tap) * cap + i] : kNone;
-  const bool valid = row != kNone;
+  const int64_t first = static_cast<int64_t>(b) * kRbChunk + threadIdx.x * kRbItems;
+  uint4 s4 = make_uint4(kNone, kNone, kNone, kNone);
+  if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<size_t>(tap) * pitch + first);
+  const uint32_t v[kRbItems] = {s4.x, s4.y, s4.z, s4.w};
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j) mine += (first + j < n && v[j] != kNone);
   uint32_t total;
-  const uint32_t rank = blockExclusiveScan(valid ? 1u : 0u, scratch, &total);
-  if (valid) {
-    gather[pos + rank] = static_cast<int32_t>(i);
-    scatter[pos + rank] = static_cast<int32_t>(row);
-    tapRow[pos + rank] = tap;
+  uint32_t at = pos + blockExclusiveScan(mine, scratch, &total);
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j) {
+    if (first + j < n && v[j] != kNone) {
+      gather[at] = static_cast<int32_t>(first + j);
+      scatter[at] = static_cast<int32_t>(v[j]);
+      tapRow[at] = tap;
+      ++at;
+    }
+  }
+}
+
+// ===========================================================================
+// Block-map path.  When the grid is small enough to afford 16 bytes per 64
+// cells, occupancy is kept in a dense table of records instead of the hash:
+//   record = { u64 bits; u32 prefix; u32 pad }   one per block of 64 cells
+// A block is a small brick of the grid (4x4x4 cells in 3-D), so a 3x3x3
+// neighbourhood touches 1-8 records, all close in memory and resident in L2,
+// where a hash probe costs one random cache line per tap.  A voxel's rank is
+// prefix + popcount(bits below its own), i.e. voxels are ranked in brick-major
+// order.  SubM looks rows up through perm[rank]; strided outputs are numbered
+// by their rank directly, which needs no CAS, no owner election, and leaves
+// output rows sorted brick-major, so neighbouring voxels sit in neighbouring
+// feature rows for the convolution's gathers.
+// ===========================================================================
+struct __attribute__((aligned(16))) BmRecord {
+  unsigned long long bits;
+  uint32_t prefix;
+  uint32_t pad;
+};
+
+struct BlockMap {
+  int shift[kMaxSpatial];  // log2 brick extent per spatial dim (extents multiply to 64)
+  int nb[kMaxSpatial];     // bricks per dim
+  uint32_t records;        // batch * product of nb
+};
+
+__device__ __forceinline__ void bmLocate(const BlockMap& m, const int c[5], uint32_t* rec, uint32_t* bit) {
+  uint32_t r = static_cast<uint32_t>(c[0]);
+  uint32_t b = 0;
+#pragma unroll
+  for (int dim = 0; dim < kMaxSpatial; ++dim) {
+    const uint32_t v = static_cast<uint32_t>(c[dim + 1]);
+    r = r * static_cast<uint32_t>(m.nb[dim]) + (v >> m.shift[dim]);
+    b = (b << m.shift[dim]) | (v & ((1u << m.shift[dim]) - 1));
+  }
+  *rec = r;
+  *bit = b;
+}
+
+// Output voxel of (input coordinate, tap) as a coordinate; false if off-lattice or outside the grid.
+__device__ __forceinline__ bool tapTargetCoord(const RbGeom& g, const int c[5], const int idx[kMaxSpatial], int o[5]) {
+  bool ok = c[0] >= 0 && c[0] < g.shape[0];
+  o[0] = c[0];
+#pragma unroll
+  for (int dim = 0; dim < kMaxSpatial; ++dim) {
+    int v = 0;
+    ok = tapDim(g, dim, c[dim + 1], idx[dim], v) && ok;
+    o[dim + 1] = v;
+  }
+  return ok;
+}
+
+__device__ __forceinline__ uint32_t bmRank(const BmRecord& r, uint32_t bit) {
+  return r.prefix + static_cast<uint32_t>(__popcll(r.bits & ((1ull << bit) - 1ull)));
+}
+
+// reset for the block-map path: records = 0, index tensor = -1, counters = 0
+__global__ void __launch_bounds__(kRbThreads)
+bmReset(uint4* records16, int64_t nRecords, int32_t* index, int64_t nIndex, uint32_t* counters, int64_t nCounters,
+        int32_t* numIndex) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
+  for (int64_t i = tid; i < nRecords; i += stride) records16[i] = zero;
+  const uintptr_t base = reinterpret_cast<uintptr_t>(index);
+  int64_t head = ((16 - (base & 15)) & 15) >> 2;
+  if (head > nIndex) head = nIndex;
+  const int64_t body16 = (nIndex - head) >> 2;
+  uint4* body = reinterpret_cast<uint4*>(index + head);
+  for (int64_t i = tid; i < body16; i += stride) body[i] = ones;
+  const int64_t tailStart = head + (body16 << 2);
+  if (tid < head) index[tid] = -1;
+  if (tid < nIndex - tailStart) index[tailStart + tid] = -1;
+  for (int64_t q = tid; q < nCounters; q += stride) counters[q] = 0;
+  if (tid == 0) *numIndex = 0;
+}
+
+// SubM: mark the input voxels.
+__global__ void __launch_bounds__(kRbThreads)
+bmMarkInputs(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
+             BmRecord* records) {
+  const int n = liveCount(numActIn, cap);
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int c[5];
+  loadCoord(coors, g.nd, i, c);
+  if (!coordInGrid(g, c)) return;
+  uint32_t rec, bit;
+  bmLocate(m, c, &rec, &bit);
+  atomicOr(&records[rec].bits, 1ull << bit);
+}
+
+// Strided / transposed: mark every candidate output (reference: convGeometryKernel, index.cu:86-102).
+// A bit that a plain read already shows set needs no atomic; bits are only ever set.
+__global__ void __launch_bounds__(kRbThreads)
+bmMarkCandidates(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn,
+                 int64_t cap, BmRecord* records) {
+  const int n = liveCount(numActIn, cap);
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
+  if (first >= n) return;
+  int idx[kMaxSpatial];
+  tapPositions(g, blockIdx.y, idx);
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j) {
+    const int64_t i = first + j;
+    if (i >= n) break;
+    int c[5], o[5];
+    loadCoord(coors, g.nd, i, c);
+    if (!tapTargetCoord(g, c, idx, o)) continue;
+    uint32_t rec, bit;
+    bmLocate(m, o, &rec, &bit);
+    const unsigned long long mask = 1ull << bit;
+    if ((__builtin_nontemporal_load(&records[rec].bits) & mask) == 0) atomicOr(&records[rec].bits, mask);
+  }
+}
+
+// Occupied cells per chunk of 1024 records.
+__global__ void __launch_bounds__(kRbThreads)
+bmChunkTotals(const BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* __restrict__ chunkTotals) {
+  __shared__ uint32_t scratch[kRbThreads / 64];
+  const uint32_t first = blockIdx.x * kRbChunk + threadIdx.x * kRbItems;
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j)
+    if (first + j < nRecords) mine += static_cast<uint32_t>(__popcll(records[first + j].bits));
+  const uint32_t total = blockSum(mine, scratch);
+  if (threadIdx.x == 0) chunkTotals[blockIdx.x] = total;
+}
+
+// Writes every record's prefix; for strided convolutions also emits the output
+// coordinates in rank order (reference: coorsOutOrganizeKernel, index.cu:104-121)
+// and numActOut = min(total, maxNumActOut).
+__global__ void __launch_bounds__(kRbThreads)
+bmPrefix(RbGeom g, BlockMap m, BmRecord* __restrict__ records, uint32_t nRecords,
+         const uint32_t* __restrict__ chunkTotals, uint32_t nChunks, int32_t* __restrict__ outCoors,
+         int32_t* numActOut, int32_t maxNumActOut) {
+  __shared__ uint32_t scratch[kRbThreads / 64];
+  uint32_t before = 0, all = 0;
+  for (uint32_t q = threadIdx.x; q < nChunks; q += blockDim.x) {
+    const uint32_t v = chunkTotals[q];
+    if (q < blockIdx.x) before += v;
+    all += v;
+  }
+  const uint32_t base = blockSum(before, scratch);
+  if (blockIdx.x == 0 && numActOut) {
+    const uint32_t total = blockSum(all, scratch);
+    if (threadIdx.x == 0)
+      *numActOut = static_cast<int32_t>(total < static_cast<uint32_t>(maxNumActOut) ? total : maxNumActOut);
+  }
+  const uint32_t first = blockIdx.x * kRbChunk + threadIdx.x * kRbItems;
+  unsigned long long bits[kRbItems];
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j) {
+    bits[j] = first + j < nRecords ? records[first + j].bits : 0ull;
+    mine += static_cast<uint32_t>(__popcll(bits[j]));
+  }
+  uint32_t total;
+  uint32_t rank = base + blockExclusiveScan(mine, scratch, &total);
+  const int cw = g.nd + 1;
+  const int pad = kMaxSpatial - g.nd;
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j) {
+    if (first + j >= nRecords) break;
+    records[first + j].prefix = rank;
+    if (outCoors && bits[j]) {
+      // brick coordinates of this record
+      uint32_t r = first + j;
+      int brick[kMaxSpatial];
+#pragma unroll
+      for (int dim = kMaxSpatial - 1; dim >= 0; --dim) {
+        brick[dim] = static_cast<int>(r % static_cast<uint32_t>(m.nb[dim])) << m.shift[dim];
+        r /= static_cast<uint32_t>(m.nb[dim]);
+      }
+      const int batch = static_cast<int>(r);
+      unsigned long long rest = bits[j];
+      uint32_t id = rank;
+      while (rest && id < static_cast<uint32_t>(maxNumActOut)) {
+        uint32_t bit = static_cast<uint32_t>(__ffsll(static_cast<long long>(rest))) - 1u;
+        rest &= rest - 1;
+        int32_t* row = outCoors + static_cast<size_t>(id) * cw;
+        row[0] = batch;
+#pragma unroll
+        for (int dim = kMaxSpatial - 1; dim >= 0; --dim) {
+          const int v = brick[dim] + static_cast<int>(bit & ((1u << m.shift[dim]) - 1));
+          bit >>= m.shift[dim];
+          if (dim >= pad) row[1 + dim - pad] = v;
+        }
+        ++id;
+      }
+    }
+    rank += static_cast<uint32_t>(__popcll(bits[j]));
+  }
+}
+
+// SubM: perm[rank of voxel i] = i (reference: the value side of setSubMHashKernel, index.cu:174-182).
+__global__ void __launch_bounds__(kRbThreads)
+bmPermutation(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn,
+              int64_t cap, const BmRecord* __restrict__ records, uint32_t* __restrict__ perm,
+              uint32_t* permShuffled) {
+  const int n = liveCount(numActIn, cap);
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int c[5];
+  loadCoord(coors, g.nd, i, c);
+  if (!coordInGrid(g, c)) return;
+  uint32_t rec, bit;
+  bmLocate(m, c, &rec, &bit);
+  const uint32_t rank = bmRank(records[rec], bit);
+  perm[rank] = static_cast<uint32_t>(i);
+  // rows that already sit in rank order (the outputs of a strided rulebook of this engine do)
+  // need no permutation lookups in the probe; any mismatch raises the flag
+  if (rank != static_cast<uint32_t>(i)) *permShuffled = 1u;
+}
+
+// SubM probe / strided resolve on the block map: staging[tap, i] = output row of
+// pair (tap, i) or ~0, plus per-(tap, chunk) counts.  For SubM the output row is
+// perm[rank]; for strided convolutions it is the rank itself, dropped when it
+// falls beyond maxNumActOut (reference: hashOutIndexKernel, index.cu:158-172).
+template <bool SUBM>
+__global__ void __launch_bounds__(kRbThreads)
+bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
+        int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ perm,
+        const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
+        uint32_t* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
+  __shared__ uint32_t scratch[kRbThreads / 64];
+  const int n = liveCount(numActIn, cap);
+  const int tap = blockIdx.y;
+  const bool shuffled = SUBM && *permShuffled != 0;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
+  uint32_t found = 0;
+  if (static_cast<int64_t>(blockIdx.x) * kRbChunk < n) {  // workgroup-uniform
+    int idx[kMaxSpatial];
+    tapPositions(g, tap, idx);
+    uint32_t row[kRbItems];
+#pragma unroll
+    for (int j = 0; j < kRbItems; ++j) {
+      row[j] = kNone;
+      const int64_t i = first + j;
+      if (i < n) {
+        int c[5], o[5];
+        loadCoord(coors, g.nd, i, c);
+        if (tapTargetCoord(g, c, idx, o)) {
+          uint32_t rec, bit;
+          bmLocate(m, o, &rec, &bit);
+          const BmRecord r = records[rec];
+          if ((r.bits >> bit) & 1ull) {
+            const uint32_t rank = bmRank(r, bit);
+            if (SUBM) {
+              row[j] = shuffled ? perm[rank] : rank;
+            } else if (rank < static_cast<uint32_t>(maxNumActOut)) {
+              row[j] = rank;
+            }
+          }
+        }
+      }
+      found += row[j] != kNone;
+    }
+    if (first < n) *reinterpret_cast<uint4*>(staging + static_cast<size_t>(tap) * pitch + first) =
+        make_uint4(row[0], row[1], row[2], row[3]);
+  }
+  publishCount(found, scratch, cnt, nBlocks, totals);
+}
+
+// ---------------------------------------------------------------------------
+// "Near" passes of the block-map path.  When, in every dim, the taps of one
+// input reach at most E+1 consecutive output cells (E = brick extent), all
+// targets of that input lie in a 2x2x2 group of bricks.  One thread then
+// serves one input: it fetches that group once (8 independent 16-byte loads,
+// neighbours in memory) and resolves all kVol taps from it, instead of one
+// random record access per (tap, input) pair.  A wavefront's memory requests
+// drop from 64 lines per tap to a handful per input, which is what bounds
+// these passes: the request rate of scattered accesses, not bandwidth.
+// Requires the outermost of the four dims to be degenerate (always true for
+// 1-D..3-D rulebooks).
+// ---------------------------------------------------------------------------
+constexpr int kNearGroup = 8;
+
+// Lowest output cell (clamped to 0) any tap of input coordinate `in` can reach in `dim`.
+__device__ __forceinline__ int nearBaseCell(const RbGeom& g, int dim, int in) {
+  if (g.transpose) {
+    const int lo = in * g.s[dim] - g.p[dim];
+    return lo > 0 ? lo : 0;
+  }
+  const int lo = in + g.p[dim] - (g.k[dim] - 1) * g.d[dim];
+  if (lo <= 0) return 0;
+  const int st = g.s[dim];
+  return st == 1 ? lo : (st == 2 ? (lo + 1) >> 1 : (lo + st - 1) / st);
+}
+
+struct NearBase {
+  int brick[kMaxSpatial];   // lower brick of the group per dim
+  uint32_t rec0;            // record index of (brick[0..3])
+  bool ok;                  // batch and dim-0 in range
+};
+
+__device__ __forceinline__ NearBase nearBase(const RbGeom& g, const BlockMap& m, const int c[5]) {
+  NearBase b;
+  b.ok = c[0] >= 0 && c[0] < g.shape[0];
+  uint32_t r = static_cast<uint32_t>(c[0]);
+#pragma unroll
+  for (int dim = 0; dim < kMaxSpatial; ++dim) {
+    b.brick[dim] = nearBaseCell(g, dim, c[dim + 1]) >> m.shift[dim];
+    r = r * static_cast<uint32_t>(m.nb[dim]) + static_cast<uint32_t>(b.brick[dim]);
+  }
+  b.rec0 = r;
+  return b;
+}
+
+// Record index offset and validity of group member e = (e1, e2, e3) in {0,1}^3.
+__device__ __forceinline__ bool nearMember(const BlockMap& m, const NearBase& b, int e, uint32_t* rec) {
+  const int e1 = (e >> 2) & 1, e2 = (e >> 1) & 1, e3 = e & 1;
+  *rec = b.rec0 + static_cast<uint32_t>((e1 * m.nb[2] + e2) * m.nb[3] + e3);
+  return b.ok && b.brick[0] < m.nb[0] && b.brick[1] + e1 < m.nb[1] && b.brick[2] + e2 < m.nb[2] &&
+         b.brick[3] + e3 < m.nb[3];
+}
+
+// Calls f(tap, valid, member, bit) for every tap of one input (dim 0 degenerate: k[0] == 1).
+template <class Fn>
+__device__ __forceinline__ void nearForEachTap(const RbGeom& g, const BlockMap& m, const int c[5], const NearBase& b,
+                                               Fn&& f) {
+  int o0;
+  const bool ok0 = b.ok && tapDim(g, 0, c[1], 0, o0);
+  int tap = 0;
+  for (int i1 = 0; i1 < g.k[1]; ++i1) {
+    int o1;
+    const bool ok1 = tapDim(g, 1, c[2], i1, o1) && ok0;
+    const int e1 = (o1 >> m.shift[1]) - b.brick[1];
+    for (int i2 = 0; i2 < g.k[2]; ++i2) {
+      int o2;
+      const bool ok2 = tapDim(g, 2, c[3], i2, o2) && ok1;
+      const int e2 = (o2 >> m.shift[2]) - b.brick[2];
+      for (int i3 = 0; i3 < g.k[3]; ++i3) {
+        int o3;
+        const bool ok3 = tapDim(g, 3, c[4], i3, o3) && ok2;
+        const int e3 = (o3 >> m.shift[3]) - b.brick[3];
+        uint32_t bit = static_cast<uint32_t>(o0) & ((1u << m.shift[0]) - 1);
+        bit = (bit << m.shift[1]) | (static_cast<uint32_t>(o1) & ((1u << m.shift[1]) - 1));
+        bit = (bit << m.shift[2]) | (static_cast<uint32_t>(o2) & ((1u << m.shift[2]) - 1));
+        bit = (bit << m.shift[3]) | (static_cast<uint32_t>(o3) & ((1u << m.shift[3]) - 1));
+        f(tap, ok3, ((e1 & 1) << 2) | ((e2 & 1) << 1) | (e3 & 1), bit);
+        ++tap;
+      }
+    }
+  }
+}
+
+// Record indices of the 8 group members; members outside the grid are clamped to record 0 (so that every
+// load is unconditional and all eight issue back to back) and reported absent in the returned mask.
+__device__ __forceinline__ uint32_t nearMembers(const BlockMap& m, const NearBase& b, uint32_t rec[kNearGroup]) {
+  uint32_t present = 0;
+#pragma unroll
+  for (int e = 0; e < kNearGroup; ++e) {
+    uint32_t r;
+    const bool ok = nearMember(m, b, e, &r);
+    rec[e] = ok ? r : 0u;
+    present |= (ok ? 1u : 0u) << e;
+  }
+  return present;
+}
+
+// Strided / transposed: one thread marks all candidate outputs of one input,
+// one atomicOr per brick of its group (and none where a read shows the bits set).
+__global__ void __launch_bounds__(kRbThreads)
+bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
+           BmRecord* records) {
+  __shared__ unsigned long long masks[kNearGroup][kRbThreads];
+  const int n = liveCount(numActIn, cap);
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kRbThreads + threadIdx.x;
+  if (i >= n) return;
+  int c[5];
+  loadCoord(coors, g.nd, i, c);
+  const NearBase b = nearBase(g, m, c);
+  uint32_t rec[kNearGroup];
+  const uint32_t present = nearMembers(m, b, rec);
+  unsigned long long have[kNearGroup];
+#pragma unroll
+  for (int e = 0; e < kNearGroup; ++e) have[e] = __builtin_nontemporal_load(&records[rec[e]].bits);
+#pragma unroll
+  for (int e = 0; e < kNearGroup; ++e) masks[e][threadIdx.x] = 0ull;
+  nearForEachTap(g, m, c, b, [&](int, bool ok, int member, uint32_t bit) {
+    if (ok) masks[member][threadIdx.x] |= 1ull << bit;
+  });
+#pragma unroll
+  for (int e = 0; e < kNearGroup; ++e) {
+    const unsigned long long want = masks[e][threadIdx.x];
+    if (((present >> e) & 1u) && (have[e] & want) != want) atomicOr(&records[rec[e]].bits, want);
+  }
+}
+
+// SubM probe / strided resolve, one thread per input (see bmProbe for the per-pair form).
+// cnt is accumulated with atomics (four workgroups share one chunk of 1024 inputs) and must start at zero.
+template <bool SUBM>
+__global__ void __launch_bounds__(kRbThreads)
+bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
+            int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ perm,
+            const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
+            uint32_t* cnt, uint32_t nBlocks, uint32_t* totals) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char nearSmem[];
+  uint4* group = reinterpret_cast<uint4*>(nearSmem);                                   // [8][kRbThreads] records
+  uint32_t* ldsCnt = reinterpret_cast<uint32_t*>(group + kNearGroup * kRbThreads);    // [kVol]
+  const int n = liveCount(numActIn, cap);
+  const int64_t i0 = static_cast<int64_t>(blockIdx.x) * kRbThreads;
+  if (i0 >= n) return;  // workgroup-uniform
+  for (int t = threadIdx.x; t < g.kVol; t += blockDim.x) ldsCnt[t] = 0;
+  const bool shuffled = SUBM && *permShuffled != 0;  // rows are not already in rank order
+  const int64_t i = i0 + threadIdx.x;
+  const bool live = i < n;
+  int c[5] = {0, 0, 0, 0, 0};
+  if (live) loadCoord(coors, g.nd, i, c);
+  const NearBase b = nearBase(g, m, c);
+  uint32_t rec[kNearGroup];
+  const uint32_t present = live ? nearMembers(m, b, rec) : (nearMembers(m, b, rec), 0u);
+  uint4 loaded[kNearGroup];
+#pragma unroll
+  for (int e = 0; e < kNearGroup; ++e) loaded[e] = *reinterpret_cast<const uint4*>(records + (live ? rec[e] : 0u));
+#pragma unroll
+  for (int e = 0; e < kNearGroup; ++e)
+    group[e * kRbThreads + threadIdx.x] = ((present >> e) & 1u) ? loaded[e] : make_uint4(0, 0, 0, 0);
+  __syncthreads();  // ldsCnt zeroed
+  nearForEachTap(g, m, c, b, [&](int tap, bool ok, int member, uint32_t bit) {
+    uint32_t row = kNone;
+    if (live && ok) {
+      const uint4 v = group[member * kRbThreads + threadIdx.x];
+      const unsigned long long bits = (static_cast<unsigned long long>(v.y) << 32) | v.x;
+      if ((bits >> bit) & 1ull) {
+        const uint32_t rank = v.z + static_cast<uint32_t>(__popcll(bits & ((1ull << bit) - 1ull)));
+        if (SUBM) {
+          row = shuffled ? perm[rank] : rank;
+        } else if (rank < static_cast<uint32_t>(maxNumActOut)) {
+          row = rank;
+        }
+      }
+    }
+    if (live) staging[static_cast<size_t>(tap) * pitch + i] = row;
+    const unsigned long long hit = __ballot(row != kNone);
+    if ((threadIdx.x & 63) == 0 && hit) atomicAdd(&ldsCnt[tap], static_cast<uint32_t>(__popcll(hit)));
+  });
+  __syncthreads();
+  const uint32_t chunk = blockIdx.x / kRbItems;
+  for (int t = threadIdx.x; t < g.kVol; t += blockDim.x) {
+    const uint32_t v = ldsCnt[t];
+    if (v) {
+      atomicAdd(&cnt[static_cast<size_t>(t) * nBlocks + chunk], v);
+      atomicAdd(&totals[t], v);
+    }
   }
 }
 
@@ -449,40 +963,123 @@ int maxCompatibleTaps(int k, int s, int d) {
 
 }  // namespace
 
-RbWorkspace planRulebookWorkspace(const RbGeom& g, int64_t cap, bool subM) {
+namespace {
+
+// Brick shape per number of real spatial dims (extents multiply to 64).
+BlockMap makeBlockMap(const RbGeom& g, uint64_t* records) {
+  static const int kShifts[kMaxSpatial + 1][kMaxSpatial] = {
+      {0, 0, 0, 6}, {0, 0, 0, 6}, {0, 0, 3, 3}, {0, 2, 2, 2}, {1, 1, 2, 2}};
+  BlockMap m{};
+  uint64_t n = static_cast<uint64_t>(g.shape[0] > 0 ? g.shape[0] : 0);
+  for (int dim = 0; dim < kMaxSpatial; ++dim) {
+    m.shift[dim] = kShifts[g.nd][dim];
+    const int extent = g.shape[dim + 1] > 0 ? g.shape[dim + 1] : 0;
+    m.nb[dim] = (extent + (1 << m.shift[dim]) - 1) >> m.shift[dim];
+    n *= static_cast<uint64_t>(m.nb[dim]);
+  }
+  *records = n;
+  m.records = static_cast<uint32_t>(n < 0xFFFFFFFFull ? n : 0xFFFFFFFFull);
+  return m;
+}
+
+constexpr uint64_t kMaxBlockMapBytes = 256ull << 20;
+
+// D3D_RULEBOOK=hash or =blockmap pins the occupancy structure (tests, tuning);
+// otherwise the block map is used whenever its records fit kMaxBlockMapBytes.
+int structureOverride() {
+  const char* e = std::getenv("D3D_RULEBOOK");
+  if (!e) return 0;
+  if (std::strcmp(e, "hash") == 0) return 1;
+  if (std::strcmp(e, "blockmap") == 0) return 2;
+  return 0;
+}
+
+RbWorkspace planWith(const RbGeom& g, int64_t cap, bool subM, bool blockMap) {
   RbWorkspace w{};
   if (cap < 1) cap = 1;
-  uint64_t bound;
-  if (subM) {
-    bound = static_cast<uint64_t>(cap);
-  } else {
-    uint64_t perInput = 1;
-    for (int dim = 0; dim < kMaxSpatial; ++dim)
-      perInput *= g.transpose ? g.k[dim] : maxCompatibleTaps(g.k[dim], g.s[dim], g.d[dim]);
-    bound = perInput * static_cast<uint64_t>(cap);
-    uint64_t cells = 1;
-    for (int dim = 0; dim <= kMaxSpatial; ++dim) cells *= static_cast<uint64_t>(g.shape[dim] > 0 ? g.shape[dim] : 1);
-    if (cells < bound) bound = cells;
-  }
-  w.slots = nextPow2(bound * 2 < 1024 ? 1024 : bound * 2);
-  w.nBlocks = static_cast<uint32_t>((cap + kRbThreads - 1) / kRbThreads);
+  w.blockMap = blockMap;
+  w.nBlocks = static_cast<uint32_t>((cap + kRbChunk - 1) / kRbChunk);
+  w.pitch = static_cast<int64_t>(w.nBlocks) * kRbChunk;
   size_t off = 0;
-  w.table = off;
-  off = alignUp(off + static_cast<size_t>(w.slots) * 8);
-  w.ids = off;
-  if (!subM) off = alignUp(off + static_cast<size_t>(w.slots) * 4);
+  if (blockMap) {
+    uint64_t records;
+    makeBlockMap(g, &records);
+    w.nRecords = static_cast<uint32_t>(records);
+    w.nChunks = static_cast<uint32_t>((records + kRbChunk - 1) / kRbChunk);
+    w.table = off;  // BmRecord [nRecords]
+    off = alignUp(off + static_cast<size_t>(records) * sizeof(BmRecord));
+    w.ids = off;    // SubM: perm u32 [cap]
+    if (subM) off = alignUp(off + static_cast<size_t>(cap) * 4);
+    w.ownCnt = off;  // chunk totals u32 [nChunks]
+    off = alignUp(off + static_cast<size_t>(w.nChunks > 0 ? w.nChunks : 1) * 4);
+  } else {
+    uint64_t bound;
+    if (subM) {
+      bound = static_cast<uint64_t>(cap);
+    } else {
+      uint64_t perInput = 1;
+      for (int dim = 0; dim < kMaxSpatial; ++dim)
+        perInput *= g.transpose ? g.k[dim] : maxCompatibleTaps(g.k[dim], g.s[dim], g.d[dim]);
+      bound = perInput * static_cast<uint64_t>(cap);
+      uint64_t cells = 1;
+      for (int dim = 0; dim <= kMaxSpatial; ++dim)
+        cells *= static_cast<uint64_t>(g.shape[dim] > 0 ? g.shape[dim] : 1);
+      if (cells < bound) bound = cells;
+    }
+    w.slots = nextPow2(bound * 2 < 1024 ? 1024 : bound * 2);
+    w.table = off;
+    off = alignUp(off + static_cast<size_t>(w.slots) * 8);
+    w.ids = off;
+    if (!subM) off = alignUp(off + static_cast<size_t>(w.slots) * 4);
+    w.ownCnt = off;
+    if (!subM) off = alignUp(off + static_cast<size_t>(g.kVol) * w.nBlocks * 4);
+  }
   w.staging = off;
-  off = alignUp(off + static_cast<size_t>(g.kVol) * cap * 4);
-  w.ownPrefix = off;
-  if (!subM) off = alignUp(off + static_cast<size_t>(cap) * 4);
-  w.blockOwn = off;
-  if (!subM) off = alignUp(off + static_cast<size_t>(w.nBlocks) * 4);
-  w.cnt = off;
-  off = alignUp(off + static_cast<size_t>(g.kVol) * w.nBlocks * 4);
-  w.totals = off;
-  off = alignUp(off + static_cast<size_t>(g.kVol) * 4);
+  off = alignUp(off + static_cast<size_t>(g.kVol) * w.pitch * 4);
+  w.cnt = off;     // [kVol, nBlocks], directly followed (no gap) by
+  off += static_cast<size_t>(g.kVol) * w.nBlocks * 4;
+  w.totals = off;  // [2, kVol] + 1: valid pairs per tap, owned outputs per tap, "rows not in rank order" flag
+  off = alignUp(off + (static_cast<size_t>(g.kVol) * 2 + 1) * 4);
   w.total = off;
   return w;
+}
+
+// True if every input's targets fall in one 2x2x2 group of bricks (see the "near" passes).
+bool nearEligible(const RbGeom& g, const BlockMap& m) {
+  if (g.k[0] != 1) return false;
+  for (int dim = 1; dim < kMaxSpatial; ++dim) {
+    const int reach = g.transpose ? (g.k[dim] - 1) * g.d[dim] : ((g.k[dim] - 1) * g.d[dim]) / g.s[dim];
+    if (reach > (1 << m.shift[dim])) return false;
+  }
+  const char* e = std::getenv("D3D_RULEBOOK_NEAR");
+  return !(e && e[0] == '0');
+}
+
+bool blockMapFits(const RbGeom& g) {
+  uint64_t records;
+  makeBlockMap(g, &records);
+  return records > 0 && records * sizeof(BmRecord) <= kMaxBlockMapBytes;
+}
+
+}  // namespace
+
+size_t rulebookWorkspaceBytes(const RbGeom& g, int64_t cap, bool subM, bool gridKnown) {
+  // enough for either structure, so the choice at enqueue time is free
+  size_t need = planWith(g, cap, subM, false).total;
+  if (gridKnown && blockMapFits(g)) {
+    const size_t bm = planWith(g, cap, subM, true).total;
+    if (bm > need) need = bm;
+  }
+  return need;
+}
+
+RbWorkspace planRulebookWorkspace(const RbGeom& g, int64_t cap, bool subM, size_t workspaceBytes) {
+  const int pin = structureOverride();
+  if (pin != 1 && blockMapFits(g)) {
+    const RbWorkspace w = planWith(g, cap, subM, true);
+    if (w.total <= workspaceBytes || pin == 2) return w;
+  }
+  return planWith(g, cap, subM, false);
 }
 
 int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const int32_t* numActIn, int64_t cap,
@@ -512,7 +1109,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       return D3D_ERR_UNSUPPORTED;
     }
   }
-  const RbWorkspace w = planRulebookWorkspace(g, cap, subM);
+  const RbWorkspace w = planRulebookWorkspace(g, cap, subM, workspaceBytes);
   if (!workspace || workspaceBytes < w.total) {
     setError("rulebook: workspace of %zu bytes, %zu needed", workspaceBytes, w.total);
     return D3D_ERR_WORKSPACE;
@@ -522,42 +1119,87 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     return D3D_ERR_BAD_ARG;
   }
   char* ws = static_cast<char*>(workspace);
-  auto* table = reinterpret_cast<unsigned long long*>(ws + w.table);
-  auto* ids = reinterpret_cast<uint32_t*>(ws + w.ids);
   auto* staging = reinterpret_cast<uint32_t*>(ws + w.staging);
-  auto* ownPrefix = reinterpret_cast<uint32_t*>(ws + w.ownPrefix);
-  auto* blockOwn = reinterpret_cast<uint32_t*>(ws + w.blockOwn);
   auto* cnt = reinterpret_cast<uint32_t*>(ws + w.cnt);
   auto* totals = reinterpret_cast<uint32_t*>(ws + w.totals);
-  const uint32_t mask = w.slots - 1;
+  uint32_t* ownTotals = totals + g.kVol;
   const int64_t rowLen = static_cast<int64_t>(g.kVol) * (cap + kSegment);
   const int64_t nIndex = 3 * rowLen;
-  const int64_t nTable16 = static_cast<int64_t>(w.slots) / 2;
-
-  // streaming fill: enough workgroups to cover the CUs several times over
-  const int64_t fillItems = nTable16 + nIndex / 4 + 1;
-  int fillBlocks = static_cast<int>((fillItems + kRbThreads - 1) / kRbThreads);
-  if (fillBlocks > 256 * 16) fillBlocks = 256 * 16;
-  if (fillBlocks < 1) fillBlocks = 1;
-  hipLaunchKernelGGL(rbReset, dim3(fillBlocks), dim3(kRbThreads), 0, stream, reinterpret_cast<uint4*>(table), nTable16,
-                     index, nIndex, totals, g.kVol, numIndex);
-
-  const dim3 grid(w.nBlocks > 0 ? w.nBlocks : 1);
   const dim3 block(kRbThreads);
-  const size_t ldsCnt = static_cast<size_t>(g.kVol) * sizeof(uint32_t);
-  if (subM) {
-    hipLaunchKernelGGL(rbSubmInsert, grid, block, 0, stream, g, coors, numActIn, cap, table, mask);
-    hipLaunchKernelGGL(rbSubmProbe, grid, block, ldsCnt, stream, g, coors, numActIn, cap, table, mask, staging, cnt,
-                       w.nBlocks, totals);
+  const int64_t inputBlocks = (cap + kRbThreads - 1) / kRbThreads;
+  const dim3 perInput(static_cast<unsigned>(inputBlocks > 0 ? inputBlocks : 1));
+  const dim3 perTap(w.nBlocks > 0 ? w.nBlocks : 1, g.kVol);
+  auto fillGrid = [](int64_t items) {
+    int64_t blocks = (items + kRbThreads - 1) / kRbThreads;
+    if (blocks > 256 * 16) blocks = 256 * 16;  // streaming fill: cover the CUs several times over
+    return dim3(static_cast<unsigned>(blocks < 1 ? 1 : blocks));
+  };
+
+  if (w.blockMap) {
+    uint64_t nRecords64;
+    const BlockMap m = makeBlockMap(g, &nRecords64);
+    auto* records = reinterpret_cast<BmRecord*>(ws + w.table);
+    auto* perm = reinterpret_cast<uint32_t*>(ws + w.ids);
+    auto* chunkTotals = reinterpret_cast<uint32_t*>(ws + w.ownCnt);
+    const dim3 perChunk(w.nChunks > 0 ? w.nChunks : 1);
+    uint32_t* permShuffled = totals + 2 * g.kVol;
+    const bool near = nearEligible(g, m);
+    const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
+    hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + nIndex / 4 + 1), block, 0, stream,
+                       reinterpret_cast<uint4*>(records), static_cast<int64_t>(w.nRecords), index, nIndex, cnt,
+                       static_cast<int64_t>(g.kVol) * w.nBlocks + 2 * g.kVol + 1, numIndex);
+    if (subM) {
+      hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
+    } else if (near) {
+      hipLaunchKernelGGL(bmMarkNear, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
+    } else {
+      hipLaunchKernelGGL(bmMarkCandidates, perTap, block, 0, stream, g, m, coors, numActIn, cap, records);
+    }
+    hipLaunchKernelGGL(bmChunkTotals, perChunk, block, 0, stream, records, w.nRecords, chunkTotals);
+    hipLaunchKernelGGL(bmPrefix, perChunk, block, 0, stream, g, m, records, w.nRecords, chunkTotals, w.nChunks,
+                       subM ? nullptr : outCoors, subM ? nullptr : numActOut, maxNumActOut);
+    if (subM)
+      hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, perm,
+                         permShuffled);
+    if (near) {
+      if (subM) {
+        hipLaunchKernelGGL(bmProbeNear<true>, perInput, block, nearLds, stream, g, m, coors, numActIn, cap,
+                           w.pitch, records, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
+      } else {
+        hipLaunchKernelGGL(bmProbeNear<false>, perInput, block, nearLds, stream, g, m, coors, numActIn, cap,
+                           w.pitch, records, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
+      }
+    } else if (subM) {
+      hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, perm,
+                         permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
+    } else {
+      hipLaunchKernelGGL(bmProbe<false>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, perm,
+                         permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
+    }
   } else {
-    hipLaunchKernelGGL(rbConvInsert, grid, block, 0, stream, g, coors, numActIn, cap, table, mask, staging);
-    hipLaunchKernelGGL(rbConvOwner, grid, block, 0, stream, g, numActIn, cap, table, staging, ownPrefix, blockOwn);
-    hipLaunchKernelGGL(rbConvAssign, grid, block, 0, stream, g, numActIn, cap, table, staging, ownPrefix, blockOwn,
-                       w.nBlocks, ids, outCoors, numActOut, maxNumActOut);
-    hipLaunchKernelGGL(rbConvResolve, grid, block, ldsCnt, stream, g, numActIn, cap, ids, staging, maxNumActOut, cnt,
-                       w.nBlocks, totals);
+    auto* table = reinterpret_cast<unsigned long long*>(ws + w.table);
+    auto* ids = reinterpret_cast<uint32_t*>(ws + w.ids);
+    auto* ownCnt = reinterpret_cast<uint32_t*>(ws + w.ownCnt);
+    const uint32_t mask = w.slots - 1;
+    const int64_t nTable16 = static_cast<int64_t>(w.slots) / 2;
+    hipLaunchKernelGGL(rbReset, fillGrid(nTable16 + nIndex / 4 + 1), block, 0, stream,
+                       reinterpret_cast<uint4*>(table), nTable16, index, nIndex, totals, 2 * g.kVol, numIndex);
+    if (subM) {
+      hipLaunchKernelGGL(rbSubmInsert, perInput, block, 0, stream, g, coors, numActIn, cap, table, mask);
+      hipLaunchKernelGGL(rbSubmProbe, perTap, block, 0, stream, g, coors, numActIn, cap, w.pitch, table, mask,
+                         staging, cnt, w.nBlocks, totals);
+    } else {
+      hipLaunchKernelGGL(rbConvInsert, perTap, block, 0, stream, g, coors, numActIn, cap, w.pitch, table, mask,
+                         staging);
+      hipLaunchKernelGGL(rbConvOwner, perTap, block, 0, stream, g, numActIn, cap, w.pitch, table, staging, ownCnt,
+                         w.nBlocks, ownTotals);
+      hipLaunchKernelGGL(rbConvAssign, perTap, block, 0, stream, g, numActIn, cap, w.pitch, table, staging, ownCnt,
+                         w.nBlocks, ownTotals, ids, outCoors, numActOut, maxNumActOut);
+      hipLaunchKernelGGL(rbConvResolve, perTap, block, 0, stream, numActIn, cap, w.pitch, ids, staging, maxNumActOut,
+                         cnt, w.nBlocks, totals);
+    }
   }
-  hipLaunchKernelGGL(rbCompact, dim3(grid.x, g.kVol), block, 0, stream, numActIn, cap, g.kVol, staging, cnt, w.nBlocks,
+  hipLaunchKernelGGL(rbCompact, perTap, block, 0, stream, numActIn, cap, w.pitch, g.kVol, staging, cnt, w.nBlocks,
                      totals, index, index + rowLen, index + 2 * rowLen, numIndex);
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;

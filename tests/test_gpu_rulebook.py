@@ -12,6 +12,16 @@ from oracle import oracle
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture(autouse=True, params=["blockmap", "blockmap-per-pair", "hash"])
+def structure(request, monkeypatch):
+    """Every case runs on every rulebook variant: the dense block map with one thread per input (default whenever
+    the map fits and a kernel's reach is at most one brick), the block map with one thread per (tap, input) pair
+    (long-reach kernels, 4-D) and the open-addressing hash (grids too large for the map)."""
+    monkeypatch.setenv("D3D_RULEBOOK", request.param.split("-")[0])
+    monkeypatch.setenv("D3D_RULEBOOK_NEAR", "0" if request.param.endswith("per-pair") else "1")
+    return request.param
+
 SUBM_CASES = [
     # (n, grid, batch, ksize, padding, dilation)
     (500, (9, 20, 18), 2, (3, 3, 3), (1, 1, 1), (1, 1, 1)),
