@@ -95,7 +95,7 @@ struct ConvArgs {
   const int32_t* nbr;     // [kVol, outRows]
   const void* zeros;      // device, >= 512 zero bytes: the row that absent neighbours gather
   int relu;
-  int tileRows;           // 0 = choose; else rows per workgroup of the MFMA kernel (64, 128 or 256)
+  int tileRows;           // 0 = choose; else rows per workgroup of the weight-streaming MFMA kernel (128, 256, 512)
 };
 
 int32_t launchConv(const ConvArgs& a, hipStream_t stream);

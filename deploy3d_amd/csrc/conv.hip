@@ -213,57 +213,76 @@ template <> struct Frag<16> { using type = u32x2; };
 // wavefront read is one contiguous, conflict-free sweep.
 //
 // RESIDENT = true : the weights of ALL taps fit in LDS.  They are loaded once
-//   in the prologue; after that every wavefront runs alone (its own active-tap
-//   list, no barriers), with the gathers of the next two taps in flight.
+//   in the prologue and shared by up to 16 wavefronts; after that every
+//   wavefront runs alone (its own list of the taps that occur among its rows,
+//   no barriers).
 // RESIDENT = false: one tap's weights at a time, double-buffered.  The slice of
 //   tap t+1 travels global -> registers -> idle LDS buffer while tap t
-//   multiplies; one barrier per tap.  Loads are issued oldest-needed-first, because the
-//   vector-memory counter retires in order: waiting for a weight slice must
-//   not drain the younger gathers behind it.
-template <class T, int CIN, int COUT, int MT, bool RESIDENT>
-__global__ void __launch_bounds__(kConvThreads)
+//   multiplies; one barrier per tap.  The weights are requested before the
+//   rows, because the vector-memory counter retires in order: waiting for a
+//   weight slice must not drain the younger gathers behind it.
+// Either way three register sets of gathered rows rotate, so the gathers of
+// taps t+1 and t+2 are in flight while tap t multiplies.  The rotation is
+// written out as three pipeline steps per loop iteration, with no branch
+// between them (the tap list is padded to a multiple of three with null taps
+// whose rows all come from the zero row), so that the compiler can neither
+// sink a gather towards its use nor has to copy a register set that is still
+// being loaded.
+template <class T, int CIN, int COUT, int MT, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
 convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
          const int32_t* __restrict__ nbr, const T* __restrict__ zeros, int kVol, int64_t inRows, int64_t outRows,
-         int relu) {
+         int relu, int tileBlocks) {
+  constexpr int THREADS = 64 * WAVES;
   constexpr int WM = 16 * MT;            // rows per wavefront
-  constexpr int TM = 4 * WM;             // rows per workgroup
+  constexpr int TM = WAVES * WM;         // rows per workgroup
   constexpr int NT = COUT / 16;          // output-channel tiles
   constexpr int KSTEP = CIN >= 32 ? 32 : 16;
   constexpr int KK = CIN / KSTEP;        // K steps per tap
   constexpr int KG = KSTEP / 4;          // elements per lane per K step
   constexpr int WFRAGS = KK * NT * 64;   // fragments (lane granules) per tap
   constexpr int WCHUNKS = CIN * COUT / 8;  // 16-byte chunks per tap
-  constexpr int WPT = (WCHUNKS + kConvThreads - 1) / kConvThreads;
+  constexpr int WPT = (WCHUNKS + THREADS - 1) / THREADS;
   using F = typename Frag<CIN>::type;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  F* wLds = reinterpret_cast<F*>(smem);  // RESIDENT: [kVol][WFRAGS]; else [2][WFRAGS]
-  int32_t* nbT = reinterpret_cast<int32_t*>(smem + static_cast<size_t>(RESIDENT ? kVol : 2) * CIN * COUT * sizeof(T));
-  int32_t* tapList = nbT + kVol * TM;    // (!RESIDENT) active taps of the tile, then their count
+  F* wLds = reinterpret_cast<F*>(smem);  // [2][WFRAGS]
+  int32_t* nbT = reinterpret_cast<int32_t*>(smem + static_cast<size_t>(2) * CIN * COUT * sizeof(T));
+  int32_t* tapList = nbT + kVol * TM;    // active taps of the tile padded with -1, then their count
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kgrp = lane >> 4;
-  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * TM;
+  // Workgroups are dealt to the 8 XCDs round-robin; handing XCD x the x-th contiguous eighth of the tiles
+  // keeps neighbouring tiles, which gather many of the same rows, behind the same L2.
+  const int perXcd = (tileBlocks + 7) / 8;
+  const int tile = (blockIdx.x & 7) * perXcd + (blockIdx.x >> 3);
+  if (tile >= tileBlocks) return;        // workgroup-uniform, before any barrier
+  const int64_t row0 = static_cast<int64_t>(tile) * TM;
   const int32_t* nb = nbT + wave * WM;   // this wavefront's columns of the [kVol][TM] neighbour tile
 
-  // neighbour tile
-  if (!RESIDENT)
-    for (int t = tid; t <= kVol; t += kConvThreads) tapList[t] = 0;
-  if (RESIDENT) {  // all weights, once
-    const u32x4* src = reinterpret_cast<const u32x4*>(wf);
-    u32x4* dst = reinterpret_cast<u32x4*>(wLds);
-    for (int e = tid; e < kVol * WCHUNKS; e += kConvThreads) dst[e] = src[e];
-  } else {
-    __syncthreads();
-  }
-  for (int e = tid; e < kVol * TM; e += kConvThreads) {
-    const int tap = e / TM, r = e % TM;
-    const int64_t row = row0 + r;
-    int32_t src = row < outRows ? nbr[static_cast<int64_t>(tap) * outRows + row] : -1;
-    if (src >= inRows) src = -1;
-    nbT[e] = src;
-    if (!RESIDENT && src >= 0) tapList[tap] = 1;
+  for (int t = tid; t < kVol + 4; t += THREADS) tapList[t] = 0;
+  __syncthreads();
+  // neighbour tile: requests first, LDS writes after, four taps at a time
+  for (int e0 = 0; e0 < kVol * TM; e0 += 4 * THREADS) {
+    int32_t v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e = e0 + q * THREADS + tid;
+      const int tap = e / TM, r = e % TM;
+      const int64_t row = row0 + r;
+      const bool ok = e < kVol * TM && row < outRows;
+      v[q] = nbr[ok ? static_cast<int64_t>(tap) * outRows + row : 0];
+      if (!ok || v[q] >= inRows) v[q] = -1;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e = e0 + q * THREADS + tid;
+      if (e < kVol * TM) {
+        nbT[e] = v[q];
+        if (v[q] >= 0) tapList[e / TM] = 1;
+      }
+    }
   }
   __syncthreads();
 
@@ -273,13 +292,13 @@ convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
 #pragma unroll
     for (int n = 0; n < NT; ++n) acc[m][n] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  // Rows without this tap read a row of zeros (one cached line for the whole device) instead of branching
-  // or selecting afterwards: nothing touches the gathered registers until the MFMAs that consume them, so
-  // the loads of a tap issue back to back and stay in flight across the MFMAs of the taps before it.
+  // Rows without this tap (and every row of a null tap, tap < 0) read a row of zeros (one cached line for the
+  // whole device) instead of branching or selecting afterwards: nothing touches the gathered registers until
+  // the MFMAs that consume them, so the loads of a tap issue back to back and stay in flight.
   auto gatherRows = [&](int tap, F (&dst)[MT][KK]) __attribute__((always_inline)) {
     int32_t src[MT];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) src[m] = nb[tap * TM + m * 16 + r16];
+    for (int m = 0; m < MT; ++m) src[m] = tap < 0 ? -1 : nb[tap * TM + m * 16 + r16];
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       const T* rowPtr = (src[m] < 0 ? zeros : in + static_cast<size_t>(src[m]) * CIN) + kgrp * KG;
@@ -307,81 +326,46 @@ convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
 
   F bufA[MT][KK], bufB[MT][KK], bufC[MT][KK];
 
-  if constexpr (RESIDENT) {
-    // taps that occur among this wavefront's rows (wavefront-uniform masks)
-    unsigned long long active[2] = {0ull, 0ull};
-    for (int tap = 0; tap < kVol; ++tap) {
-      bool any = false;
-      for (int r = lane; r < WM; r += 64) any = any || nb[tap * TM + r] >= 0;
-      if (__ballot(any)) active[tap >> 6] |= 1ull << (tap & 63);
-    }
-    auto nextTap = [&]() __attribute__((always_inline)) -> int {
-      if (active[0]) {
-        const int t = __builtin_ctzll(active[0]);
-        active[0] &= active[0] - 1;
-        return t;
-      }
-      if (active[1]) {
-        const int t = __builtin_ctzll(active[1]);
-        active[1] &= active[1] - 1;
-        return 64 + t;
-      }
-      return -1;
-    };
-    // Three register sets: while tap t multiplies, the gathers of t+1 and t+2 are in flight.  The sets
-    // rotate through loop-carried copies, which pins each gather to the iteration that issues it.  Past
-    // the last tap the pipeline re-gathers the last tap (harmless, cached) instead of branching.
-    int tNow = nextTap();
-    if (tNow >= 0) {
-      int last = tNow;
-      int tNext = nextTap();
-      gatherRows(tNow, bufA);
-      gatherRows(tNext >= 0 ? (last = tNext) : last, bufB);
-      while (tNow >= 0) {
-        const int tFuture = nextTap();
-        gatherRows(tFuture >= 0 ? (last = tFuture) : last, bufC);
-        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMAs they are meant to overlap
-        multiply(wLds + static_cast<size_t>(tNow) * WFRAGS, bufA);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-#pragma unroll
-          for (int kk = 0; kk < KK; ++kk) {
-            bufA[m][kk] = bufB[m][kk];
-            bufB[m][kk] = bufC[m][kk];
-          }
-        tNow = tNext;
-        tNext = tFuture;
-      }
-    }
-  } else {
+  {
     if (tid == 0) {  // compact the flags into a list in place (slot n <= t is written after flag t was read)
       int n = 0;
       for (int t = 0; t < kVol; ++t)
         if (tapList[t]) tapList[n++] = t;
-      tapList[kVol] = n;
+      const int count = n;
+      while (n < kVol + 3) tapList[n++] = -1;  // null taps pad the list
+      tapList[kVol + 3] = count;
     }
     __syncthreads();
-    const int nActive = tapList[kVol];
+    const int nActive = tapList[kVol + 3];
     if (nActive > 0) {
-      // indices past the end of the list are clamped to the last tap: the pipeline then re-requests data it
-      // already has (cache hits) instead of branching around loads, which keeps every load unconditional
-      auto tapAt = [&](int a) __attribute__((always_inline)) { return tapList[a < nActive ? a : nActive - 1]; };
+      auto tapAt = [&](int a) __attribute__((always_inline)) { return tapList[a < kVol + 3 ? a : kVol + 2]; };
       auto loadWeights = [&](int a, u32x4 (&dst)[WPT]) __attribute__((always_inline)) {
-        const u32x4* wk = reinterpret_cast<const u32x4*>(wf + static_cast<size_t>(tapAt(a)) * CIN * COUT);
+        const int t = tapAt(a);
+        const u32x4* wk = reinterpret_cast<const u32x4*>(wf + static_cast<size_t>(t < 0 ? 0 : t) * CIN * COUT);
 #pragma unroll
         for (int q = 0; q < WPT; ++q) {
-          const int e = tid + q * kConvThreads;
-          dst[q] = wk[(WCHUNKS % kConvThreads == 0 || e < WCHUNKS) ? e : 0];
+          const int e = tid + q * THREADS;
+          dst[q] = wk[(WCHUNKS % THREADS == 0 || e < WCHUNKS) ? e : 0];
         }
       };
       auto storeWeights = [&](int buf, const u32x4 (&src)[WPT]) __attribute__((always_inline)) {
         u32x4* dst = reinterpret_cast<u32x4*>(wLds + buf * WFRAGS);
 #pragma unroll
         for (int q = 0; q < WPT; ++q) {
-          const int e = tid + q * kConvThreads;
-          if (WCHUNKS % kConvThreads == 0 || e < WCHUNKS) dst[e] = src[q];
+          const int e = tid + q * THREADS;
+          if (WCHUNKS % THREADS == 0 || e < WCHUNKS) dst[e] = src[q];
         }
+      };
+      // one pipeline step: tap a multiplies while the weights of a+1 and the rows of a+2 are requested
+      auto step = [&](int a, const F (&rowsNow)[MT][KK], F (&rowsFuture)[MT][KK]) __attribute__((always_inline)) {
+        u32x4 wreg[WPT];
+        loadWeights(a + 1, wreg);
+        gatherRows(tapAt(a + 2), rowsFuture);
+        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMAs they are meant to overlap
+        multiply(wLds + (a & 1) * WFRAGS, rowsNow);
+        __builtin_amdgcn_sched_barrier(0);
+        storeWeights((a + 1) & 1, wreg);
+        __syncthreads();
       };
       {
         u32x4 wreg[WPT];
@@ -391,25 +375,10 @@ convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
         storeWeights(0, wreg);
       }
       __syncthreads();
-      // One tap per iteration: tap a multiplies while the weights of a+1 and the rows of a+2 are requested.
-      // The weights are requested first, so waiting for them leaves the younger gathers in flight; the row
-      // sets rotate through loop-carried copies, which pins each gather to the iteration that issues it.
-      for (int a = 0; a < nActive; ++a) {
-        u32x4 wreg[WPT];
-        loadWeights(a + 1, wreg);
-        gatherRows(tapAt(a + 2), bufC);
-        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMAs they are meant to overlap
-        multiply(wLds + (a & 1) * WFRAGS, bufA);
-        __builtin_amdgcn_sched_barrier(0);
-        storeWeights((a + 1) & 1, wreg);
-        __syncthreads();
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-#pragma unroll
-          for (int kk = 0; kk < KK; ++kk) {
-            bufA[m][kk] = bufB[m][kk];
-            bufB[m][kk] = bufC[m][kk];
-          }
+      for (int a = 0; a < nActive; a += 3) {  // steps past nActive work on null taps: zero rows, no effect
+        step(a, bufA, bufC);
+        step(a + 1, bufB, bufA);
+        step(a + 2, bufC, bufB);
       }
     }
   }
@@ -434,58 +403,240 @@ convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
   }
 }
 
+// Small layers: the weights of ALL taps fit in LDS.  A workgroup loads them once and then lives on: each of
+// its wavefronts walks, on its own, over groups of 16 output rows (group index strided by the number of
+// wavefronts in the grid), with a private slice of the neighbour table, its own list of the taps that occur
+// in the group, and no barrier after the weight load.
+template <class T, int CIN, int COUT, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf,
+                 const float* __restrict__ bias, const int32_t* __restrict__ nbr, const T* __restrict__ zeros,
+                 int kVol, int64_t inRows, int64_t outRows, int relu, int groups) {
+  constexpr int THREADS = 64 * WAVES;
+  constexpr int MT = 1;
+  constexpr int NT = COUT / 16;
+  constexpr int KSTEP = CIN >= 32 ? 32 : 16;
+  constexpr int KK = CIN / KSTEP;
+  constexpr int KG = KSTEP / 4;
+  constexpr int WFRAGS = KK * NT * 64;
+  constexpr int WCHUNKS = CIN * COUT / 8;
+  using F = typename Frag<CIN>::type;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  F* wLds = reinterpret_cast<F*>(smem);                                              // [kVol][WFRAGS]
+  int32_t* nbAll = reinterpret_cast<int32_t*>(smem + static_cast<size_t>(kVol) * CIN * COUT * sizeof(T));
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kgrp = lane >> 4;
+  int32_t* nb = nbAll + wave * kVol * 16;                                            // [kVol][16], private
+
+  {
+    const u32x4* src = reinterpret_cast<const u32x4*>(wf);
+    u32x4* dst = reinterpret_cast<u32x4*>(wLds);
+    for (int e = tid; e < kVol * WCHUNKS; e += THREADS) dst[e] = src[e];
+  }
+  __syncthreads();
+
+  auto gatherRows = [&](int tap, F (&dst)[MT][KK]) __attribute__((always_inline)) {
+    const int32_t src = tap < 0 ? -1 : nb[tap * 16 + r16];
+    const T* rowPtr = (src < 0 ? zeros : in + static_cast<size_t>(src) * CIN) + kgrp * KG;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) dst[0][kk] = *reinterpret_cast<const F*>(rowPtr + kk * KSTEP);
+  };
+
+  // Workgroups are dealt to the 8 XCDs round-robin; XCD x takes the x-th contiguous eighth of the row groups,
+  // so neighbouring groups, which gather many of the same rows, meet behind the same L2.
+  const int wavesPerXcd = (gridDim.x / 8) * WAVES;
+  const int perXcd = (groups + 7) / 8;
+  const int xcd = blockIdx.x & 7;
+  for (int local = (blockIdx.x >> 3) * WAVES + wave; local < perXcd; local += wavesPerXcd) {
+    const int group = xcd * perXcd + local;
+    if (group >= groups) break;
+    const int64_t row0 = static_cast<int64_t>(group) * 16;
+
+    // private neighbour slice and the taps that occur in it (wavefront-uniform masks)
+    unsigned long long active[2] = {0ull, 0ull};
+    for (int t0 = 0; t0 < kVol; t0 += 4) {
+      const int tap = t0 + kgrp;
+      const int64_t row = row0 + r16;
+      const bool ok = tap < kVol && row < outRows;
+      int32_t v = nbr[ok ? static_cast<int64_t>(tap) * outRows + row : 0];
+      if (!ok || v >= inRows) v = -1;
+      if (tap < kVol) nb[tap * 16 + r16] = v;
+      const unsigned long long hit = __ballot(v >= 0);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if ((hit >> (16 * q)) & 0xFFFFull) active[(t0 + q) >> 6] |= 1ull << ((t0 + q) & 63);
+    }
+    auto nextTap = [&]() __attribute__((always_inline)) -> int {  // -1 once the list is exhausted
+      if (active[0]) {
+        const int t = __builtin_ctzll(active[0]);
+        active[0] &= active[0] - 1;
+        return t;
+      }
+      if (active[1]) {
+        const int t = __builtin_ctzll(active[1]);
+        active[1] &= active[1] - 1;
+        return 64 + t;
+      }
+      return -1;
+    };
+    auto weightsOf = [&](int tap) __attribute__((always_inline)) {
+      return wLds + static_cast<size_t>(tap < 0 ? 0 : tap) * WFRAGS;  // a null tap multiplies zero rows
+    };
+
+    float4v acc[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) acc[n] = float4v{0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const F* wTap, const F (&rows)[MT][KK]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+          const F wfrag = wTap[(kk * NT + n) * 64 + lane];
+          if constexpr (CIN >= 32) {
+            acc[n] = Mfma<T>::k32(wfrag, rows[0][kk], acc[n]);
+          } else {
+            acc[n] = Mfma<T>::k16(wfrag, rows[0][kk], acc[n]);
+          }
+        }
+      }
+    };
+
+    F bufA[MT][KK], bufB[MT][KK], bufC[MT][KK];
+    int tA = nextTap(), tB = nextTap(), tC;
+    gatherRows(tA, bufA);
+    gatherRows(tB, bufB);
+    while (tA >= 0) {  // three steps per iteration, no branch between them (see convMfma)
+      tC = nextTap();
+      gatherRows(tC, bufC);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(weightsOf(tA), bufA);
+      __builtin_amdgcn_sched_barrier(0);
+      tA = nextTap();
+      gatherRows(tA, bufA);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(weightsOf(tB), bufB);
+      __builtin_amdgcn_sched_barrier(0);
+      tB = nextTap();
+      gatherRows(tB, bufB);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(weightsOf(tC), bufC);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    const int64_t row = row0 + r16;
+    if (row < outRows) {
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        const int col = n * 16 + kgrp * 4;
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[j] = acc[n][j] + (bias ? bias[col + j] : 0.f);
+          if (relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
+        }
+        T packed[4] = {static_cast<T>(v[0]), static_cast<T>(v[1]), static_cast<T>(v[2]), static_cast<T>(v[3])};
+        *reinterpret_cast<u32x2*>(out + static_cast<size_t>(row) * COUT + col) = __builtin_bit_cast(u32x2, packed);
+      }
+    }
+  }
+}
+
 constexpr size_t kLdsLimit = 160 * 1024;
 
-template <class T, int CIN, int COUT, int MT, bool RESIDENT>
+template <int CIN, int COUT>
+constexpr size_t mfmaLds(int kVol, int rows, size_t elem) {
+  return static_cast<size_t>(2) * CIN * COUT * elem + static_cast<size_t>(kVol) * rows * 4 +
+         (static_cast<size_t>(kVol) + 4) * 4;
+}
+
+template <class K>
+int32_t grantLds(K kernel, size_t lds, size_t* granted) {
+  if (lds > *granted) {  // dynamic LDS beyond 64 KiB has to be requested per kernel
+    D3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(kLdsLimit)));
+    *granted = kLdsLimit;
+  }
+  return D3D_OK;
+}
+
+template <class T, int CIN, int COUT, int MT, int WAVES>
 int32_t launchMfmaTile(const ConvArgs& a, hipStream_t stream) {
-  constexpr int TM = 64 * MT;
-  const size_t lds = static_cast<size_t>(RESIDENT ? a.kVol : 2) * CIN * COUT * sizeof(T) +
-                     static_cast<size_t>(a.kVol) * TM * sizeof(int32_t) + (static_cast<size_t>(a.kVol) + 1) * 4;
+  constexpr int TM = 16 * MT * WAVES;
+  const size_t lds = mfmaLds<CIN, COUT>(a.kVol, TM, sizeof(T));
   if (lds > kLdsLimit) {
     setError("conv: kernel volume %d too large for the MFMA kernel", a.kVol);
     return D3D_ERR_UNSUPPORTED;
   }
-  static size_t granted = 64 * 1024;  // dynamic LDS beyond 64 KiB has to be requested per kernel
-  if (lds > granted) {
-    D3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&convMfma<T, CIN, COUT, MT, RESIDENT>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsLimit)));
-    granted = kLdsLimit;
-  }
-  const dim3 grid(static_cast<unsigned>((a.outRows + TM - 1) / TM));
-  hipLaunchKernelGGL((convMfma<T, CIN, COUT, MT, RESIDENT>), grid, dim3(kConvThreads), lds, stream,
-                     static_cast<const T*>(a.in), static_cast<T*>(a.out), static_cast<const T*>(a.weightsMfma), a.bias,
-                     a.nbr, static_cast<const T*>(a.zeros), a.kVol, a.inRows, a.outRows, a.relu);
+  static size_t granted = 64 * 1024;
+  const int32_t rc = grantLds(&convMfma<T, CIN, COUT, MT, WAVES>, lds, &granted);
+  if (rc != D3D_OK) return rc;
+  const int tiles = static_cast<int>((a.outRows + TM - 1) / TM);
+  const int perXcd = (tiles + 7) / 8;
+  hipLaunchKernelGGL((convMfma<T, CIN, COUT, MT, WAVES>), dim3(static_cast<unsigned>(perXcd * 8)), dim3(64 * WAVES),
+                     lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
+                     static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, static_cast<const T*>(a.zeros), a.kVol,
+                     a.inRows, a.outRows, a.relu, tiles);
   return D3D_OK;
 }
 
-// Rows per wavefront (16*MT): more rows amortise the weight fragments over more MFMAs; fewer rows give
-// more workgroups per CU to hide the gather latency and to fill 256 CUs.
+template <class T, int CIN, int COUT>
+int32_t launchMfmaResident(const ConvArgs& a, hipStream_t stream) {
+  constexpr int WAVES = 16;
+  const size_t lds = static_cast<size_t>(a.kVol) * CIN * COUT * sizeof(T) + static_cast<size_t>(WAVES) * a.kVol * 16 * 4;
+  static size_t granted = 64 * 1024;
+  const int32_t rc = grantLds(&convMfmaResident<T, CIN, COUT, WAVES>, lds, &granted);
+  if (rc != D3D_OK) return rc;
+  const int groups = static_cast<int>((a.outRows + 15) / 16);
+  // persistent workgroups: as many as fit on the 256 CUs at this LDS footprint, but no more than there is work
+  int perCu = static_cast<int>(kLdsLimit / (lds + 1024));
+  if (perCu < 1) perCu = 1;
+  if (perCu > 2) perCu = 2;  // 16 wavefronts each
+  int blocks = 256 * perCu;
+  const int needed = (groups + WAVES - 1) / WAVES;
+  if (blocks > needed) blocks = (needed + 7) / 8 * 8;
+  if (blocks < 8) blocks = 8;
+  hipLaunchKernelGGL((convMfmaResident<T, CIN, COUT, WAVES>), dim3(static_cast<unsigned>(blocks)), dim3(64 * WAVES),
+                     lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
+                     static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, static_cast<const T*>(a.zeros), a.kVol,
+                     a.inRows, a.outRows, a.relu, groups);
+  return D3D_OK;
+}
+
+// Small layers keep every tap's weights in LDS (convMfmaResident).  Large layers stream one tap's weights at a
+// time through LDS for 8 (or 4) wavefronts; more rows per wavefront (MT) amortise that stream.
 template <class T, int CIN, int COUT>
 int32_t launchMfmaOne(const ConvArgs& a, hipStream_t stream) {
   const size_t allTaps = static_cast<size_t>(a.kVol) * CIN * COUT * sizeof(T);
-  const bool resident = allTaps <= 56 * 1024 && a.kVol <= 128;
-  int mt = resident ? 2 : 4;
-  if (a.tileRows > 0) {
-    mt = a.tileRows / 64;
+  if (allTaps <= 56 * 1024 && a.kVol <= 128 && allTaps + static_cast<size_t>(16) * a.kVol * 16 * 4 <= kLdsLimit)
+    return launchMfmaResident<T, CIN, COUT>(a, stream);
+  // rows per workgroup = 16 * MT * WAVES
+  int mt = 2;
+  int waves = 8;
+  if (a.tileRows > 0) {  // tuning / test override: tileRows = 16 * MT * WAVES, waves encoded in bit 30
+    waves = (a.tileRows & (1 << 30)) ? 4 : 8;
+    mt = (a.tileRows & 0xFFFF) / (16 * waves);
+    if (mt < 1) mt = 1;
+    if (mt > 4) mt = 4;
+    if (mt == 3) mt = 2;
+    if (mt == 4 && CIN * COUT >= 64 * 128) mt = 2;  // would spill registers
   } else {
-    while (mt > 1 && (a.outRows + 64 * mt - 1) / (64 * mt) < 512) mt >>= 1;
+    // keep at least two workgroups per CU when the layer is small
+    while (mt > 1 && (a.outRows + 16 * mt * waves - 1) / (16 * mt * waves) < 512) mt >>= 1;
   }
-  auto ldsFor = [&](int m) {
-    return (resident ? allTaps : 2 * static_cast<size_t>(CIN) * COUT * sizeof(T)) +
-           static_cast<size_t>(a.kVol) * 64 * m * 4 + (static_cast<size_t>(a.kVol) + 1) * 4;
-  };
-  while (mt > 1 && ldsFor(mt) > kLdsLimit) mt >>= 1;
-  if (resident) {
+  while (mt > 1 && mfmaLds<CIN, COUT>(a.kVol, 16 * mt * waves, sizeof(T)) > kLdsLimit) mt >>= 1;
+  if (waves == 4) {
     switch (mt) {
-      case 4: return launchMfmaTile<T, CIN, COUT, 4, true>(a, stream);
-      case 2: return launchMfmaTile<T, CIN, COUT, 2, true>(a, stream);
-      default: return launchMfmaTile<T, CIN, COUT, 1, true>(a, stream);
+      case 4: return launchMfmaTile<T, CIN, COUT, 4, 4>(a, stream);
+      case 2: return launchMfmaTile<T, CIN, COUT, 2, 4>(a, stream);
+      default: return launchMfmaTile<T, CIN, COUT, 1, 4>(a, stream);
     }
   }
   switch (mt) {
-    case 4: return launchMfmaTile<T, CIN, COUT, 4, false>(a, stream);
-    case 2: return launchMfmaTile<T, CIN, COUT, 2, false>(a, stream);
-    default: return launchMfmaTile<T, CIN, COUT, 1, false>(a, stream);
+    case 4: return launchMfmaTile<T, CIN, COUT, 4, 8>(a, stream);
+    case 2: return launchMfmaTile<T, CIN, COUT, 2, 8>(a, stream);
+    default: return launchMfmaTile<T, CIN, COUT, 1, 8>(a, stream);
   }
 }
 

@@ -445,13 +445,15 @@ const void* zeroRow() {
   return buf->ptr;
 }
 
-// Tuning / test hook: D3D_CONV_TILE_ROWS = 64, 128 or 256 pins the rows per
-// workgroup of the MFMA convolution; unset or anything else = heuristic.
+// Tuning / test hook: D3D_CONV_TILE_ROWS = rows per workgroup of the weight-streaming MFMA convolution
+// (64 .. 512, a multiple of 64), D3D_CONV_WAVES = 4 or 8 wavefronts per workgroup; unset = heuristic.
 int tileRowsOverride() {
   const char* e = std::getenv("D3D_CONV_TILE_ROWS");
   if (!e) return 0;
   const int v = std::atoi(e);
-  return (v == 64 || v == 128 || v == 256) ? v : 0;
+  if (v < 64 || v > 512 || v % 64) return 0;
+  const char* w = std::getenv("D3D_CONV_WAVES");
+  return v | ((w && std::atoi(w) == 4) ? (1 << 30) : 0);
 }
 
 // --- SPConvMM ----------------------------------------------------------------

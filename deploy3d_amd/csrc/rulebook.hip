@@ -620,13 +620,10 @@ bmChunkTotals(const BmRecord* __restrict__ records, uint32_t nRecords, uint32_t*
   if (threadIdx.x == 0) chunkTotals[blockIdx.x] = total;
 }
 
-// Writes every record's prefix; for strided convolutions also emits the output
-// coordinates in rank order (reference: coorsOutOrganizeKernel, index.cu:104-121)
-// and numActOut = min(total, maxNumActOut).
+// Writes every record's prefix, and numActOut = min(total, maxNumActOut) for strided convolutions.
 __global__ void __launch_bounds__(kRbThreads)
-bmPrefix(RbGeom g, BlockMap m, BmRecord* __restrict__ records, uint32_t nRecords,
-         const uint32_t* __restrict__ chunkTotals, uint32_t nChunks, int32_t* __restrict__ outCoors,
-         int32_t* numActOut, int32_t maxNumActOut) {
+bmPrefix(BmRecord* __restrict__ records, uint32_t nRecords, const uint32_t* __restrict__ chunkTotals,
+         uint32_t nChunks, int32_t* numActOut, int32_t maxNumActOut) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   uint32_t before = 0, all = 0;
   for (uint32_t q = threadIdx.x; q < nChunks; q += blockDim.x) {
@@ -641,49 +638,47 @@ bmPrefix(RbGeom g, BlockMap m, BmRecord* __restrict__ records, uint32_t nRecords
       *numActOut = static_cast<int32_t>(total < static_cast<uint32_t>(maxNumActOut) ? total : maxNumActOut);
   }
   const uint32_t first = blockIdx.x * kRbChunk + threadIdx.x * kRbItems;
-  unsigned long long bits[kRbItems];
+  uint32_t count[kRbItems];
   uint32_t mine = 0;
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
-    bits[j] = first + j < nRecords ? records[first + j].bits : 0ull;
-    mine += static_cast<uint32_t>(__popcll(bits[j]));
+    count[j] = first + j < nRecords ? static_cast<uint32_t>(__popcll(records[first + j].bits)) : 0u;
+    mine += count[j];
   }
   uint32_t total;
   uint32_t rank = base + blockExclusiveScan(mine, scratch, &total);
-  const int cw = g.nd + 1;
-  const int pad = kMaxSpatial - g.nd;
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
-    if (first + j >= nRecords) break;
-    records[first + j].prefix = rank;
-    if (outCoors && bits[j]) {
-      // brick coordinates of this record
-      uint32_t r = first + j;
-      int brick[kMaxSpatial];
-#pragma unroll
-      for (int dim = kMaxSpatial - 1; dim >= 0; --dim) {
-        brick[dim] = static_cast<int>(r % static_cast<uint32_t>(m.nb[dim])) << m.shift[dim];
-        r /= static_cast<uint32_t>(m.nb[dim]);
-      }
-      const int batch = static_cast<int>(r);
-      unsigned long long rest = bits[j];
-      uint32_t id = rank;
-      while (rest && id < static_cast<uint32_t>(maxNumActOut)) {
-        uint32_t bit = static_cast<uint32_t>(__ffsll(static_cast<long long>(rest))) - 1u;
-        rest &= rest - 1;
-        int32_t* row = outCoors + static_cast<size_t>(id) * cw;
-        row[0] = batch;
-#pragma unroll
-        for (int dim = kMaxSpatial - 1; dim >= 0; --dim) {
-          const int v = brick[dim] + static_cast<int>(bit & ((1u << m.shift[dim]) - 1));
-          bit >>= m.shift[dim];
-          if (dim >= pad) row[1 + dim - pad] = v;
-        }
-        ++id;
-      }
-    }
-    rank += static_cast<uint32_t>(__popcll(bits[j]));
+    if (first + j < nRecords) records[first + j].prefix = rank;
+    rank += count[j];
   }
+}
+
+// Strided convolutions: output coordinates in rank order (reference: coorsOutOrganizeKernel,
+// index.cu:104-121).  One wavefront per record, one lane per cell of the brick.
+__global__ void __launch_bounds__(kRbThreads)
+bmEmitCoords(RbGeom g, BlockMap m, const BmRecord* __restrict__ records, uint32_t nRecords,
+             int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
+  const uint32_t rec = blockIdx.x * (kRbThreads / 64) + (threadIdx.x >> 6);
+  if (rec >= nRecords) return;
+  const BmRecord r = records[rec];
+  uint32_t bit = threadIdx.x & 63;
+  if (!((r.bits >> bit) & 1ull)) return;
+  const uint32_t id = bmRank(r, bit);
+  if (id >= static_cast<uint32_t>(maxNumActOut)) return;
+  const int pad = kMaxSpatial - g.nd;
+  int32_t* row = outCoors + static_cast<size_t>(id) * (g.nd + 1);
+  uint32_t q = rec;
+#pragma unroll
+  for (int dim = kMaxSpatial - 1; dim >= 0; --dim) {
+    const uint32_t nb = static_cast<uint32_t>(m.nb[dim]);
+    const uint32_t brick = q % nb;
+    q /= nb;
+    const int v = static_cast<int>((brick << m.shift[dim]) + (bit & ((1u << m.shift[dim]) - 1)));
+    bit >>= m.shift[dim];
+    if (dim >= pad) row[1 + dim - pad] = v;
+  }
+  row[0] = static_cast<int32_t>(q);
 }
 
 // SubM: perm[rank of voxel i] = i (reference: the value side of setSubMHashKernel, index.cu:174-182).
@@ -1156,8 +1151,11 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       hipLaunchKernelGGL(bmMarkCandidates, perTap, block, 0, stream, g, m, coors, numActIn, cap, records);
     }
     hipLaunchKernelGGL(bmChunkTotals, perChunk, block, 0, stream, records, w.nRecords, chunkTotals);
-    hipLaunchKernelGGL(bmPrefix, perChunk, block, 0, stream, g, m, records, w.nRecords, chunkTotals, w.nChunks,
-                       subM ? nullptr : outCoors, subM ? nullptr : numActOut, maxNumActOut);
+    hipLaunchKernelGGL(bmPrefix, perChunk, block, 0, stream, records, w.nRecords, chunkTotals, w.nChunks,
+                       subM ? nullptr : numActOut, maxNumActOut);
+    if (!subM)
+      hipLaunchKernelGGL(bmEmitCoords, dim3((w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64)), block, 0, stream,
+                         g, m, records, w.nRecords, outCoors, maxNumActOut);
     if (subM)
       hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, perm,
                          permShuffled);

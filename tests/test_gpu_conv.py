@@ -102,8 +102,8 @@ def test_kernel_shapes(engine, ksize, padding):
     run_case(2500, (10, 36, 30), ksize, (1, 1, 1), padding, 32, 64, "float16", True)
 
 
-@pytest.mark.parametrize("tile_rows", [64, 128, 256])
-@pytest.mark.parametrize("cin,cout", [(16, 16), (32, 64), (64, 64), (128, 128)])
+@pytest.mark.parametrize("tile_rows", [128, 256, 512])
+@pytest.mark.parametrize("cin,cout", [(32, 64), (64, 64), (64, 128), (128, 128)])
 def test_mfma_tile_sizes(engine, monkeypatch, tile_rows, cin, cout):
     """Every workgroup tile height of the MFMA kernel (the launcher normally picks one from the row count)."""
     monkeypatch.setenv("D3D_CONV_TILE_ROWS", str(tile_rows))
