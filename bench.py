@@ -20,6 +20,10 @@ sys.path.insert(0, ROOT)
 METRIC = "sparse backbone latency ms + effective TFLOP/s, 120k voxels fp16, 1×MI355X"
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the roofline kernel at the default 120 000 voxels, from two `rocprofv3 --pmc` runs of this
+# script (FETCH_SIZE 33623, WRITE_SIZE 32778 per dispatch), each scaled by what the same counter read for the
+# 256 MiB copy of --pmc-copy-mib (FETCH_SIZE reads half the copied KiB: factor 2.0; WRITE_SIZE factor 1.0).
+MEASURED_TRAFFIC_BYTES = {("conv3", 120000): int((33623 * 2.0 + 32778 * 1.0) * 1024)}
 
 
 def cpu_baseline(cfg, threads):
@@ -69,6 +73,9 @@ def main():
     ap.add_argument("--voxels", type=int, default=120000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager enqueues instead of HIP-graph replays")
+    ap.add_argument("--pmc-copy-mib", type=int, default=0,
+                    help="end with ONE device-to-device copy of this many MiB: the dispatch of known size that scales "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this script")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the sparse backbone is a single-GPU inference path); "
@@ -151,6 +158,12 @@ def main():
             ms = (time.perf_counter() - t0) * 1e3 / args.steps
             mode = "hip-graph replay"
         same = bool(torch.equal(y.feats, ref_out))
+        if args.pmc_copy_mib:
+            src = torch.ones(args.pmc_copy_mib << 20, dtype=torch.uint8, device="cuda")
+            dst = torch.empty_like(src)
+            stream.synchronize()
+            dst.copy_(src)
+            stream.synchronize()
 
     # dominant kernel: the convolution with the largest event time among layers that reuse a cached
     # neighbour table (their enqueue launches exactly one kernel)
@@ -164,7 +177,8 @@ def main():
     roofline = {
         "kernel": "convMfma<fp16,%d,%d> (layer %s)" % (dspec["cin"], dspec["cout"], dspec["name"]),
         "bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None,
+        "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
+        "traffic": MEASURED_TRAFFIC_BYTES.get((dspec["name"][:5], args.voxels)),
         "flops_per_launch": layer_flops[dom], "avg_launch_ms": round(layer_ms[dom], 4),
     }
 
