@@ -9,7 +9,7 @@
 // legally produce.  Only tests/, the smoke check and the benchmark's
 // cpu_baseline leg may load it; the shipped library never does.
 //
-// What pins each function (see tests/test_oracle_*.py):
+// What pins each function (tests/test_oracle_pins.py, tests/test_golden.py):
 //   out_shape      closed form; torch conv3d / conv_transpose3d output shapes
 //   fmix32         published MurmurHash3 finaliser known answers
 //   rulebook       brute-force dict rulebook on random clouds; the structural
