@@ -96,6 +96,7 @@ struct ConvArgs {
   const void* zeros;      // device, >= 512 zero bytes: the row that absent neighbours gather
   int relu;
   int tileRows;           // 0 = choose; else rows per workgroup of the weight-streaming MFMA kernel (128, 256, 512)
+  int staged;             // staged MFMA kernel: 0 = choose, -1 = do not use it, else MT | WAVES << 8 | NS << 16 | resident << 24
 };
 
 int32_t launchConv(const ConvArgs& a, hipStream_t stream);

@@ -543,6 +543,273 @@ convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restr
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// Staged MFMA convolution.
+//
+// A lane of the MFMA operand layout owns ONE row (lane % 16), so gathering rows
+// straight into operand registers makes adjacent lanes touch different rows, and
+// the texture path then serves 16 bytes per clock per CU.  It serves 64 when
+// the lanes of a quad read 64 contiguous bytes.  Here the gather therefore uses
+// the memory-friendly mapping (consecutive lanes sweep one row, 16 bytes each)
+// and lands in LDS without passing through registers (global_load_lds); the
+// MFMA fragments are then read from LDS in operand layout.  The 16-byte chunks
+// of a staged row are XOR-swizzled by row so both sides are conflict-free.
+//
+// Per wavefront: WM = 16*MT output rows, NS stage slots (rows of tap a+NS are
+// in flight while tap a multiplies), the neighbour indices of a tap arrive in
+// LDS the same way three taps earlier.  All vector-memory traffic of the loop
+// is asynchronous and retires in order, so one s_waitcnt vmcnt(X) per tap, X =
+// the loads that may stay in flight, is the only wait.
+//
+// Weights: RESIDENT = every tap's fragments stay in LDS (small layers, no
+// barrier at all); otherwise three tap buffers rotate (tap a multiplies, a+1
+// has landed, a+2 is landing) with one barrier per tap.
+// The result goes back through the wavefront's stage area so that rows leave
+// as whole contiguous lines.
+// ---------------------------------------------------------------------------
+template <int CH> __device__ __forceinline__ int stageSwizzle(int n) {
+  if (CH == 2) return (n >> 2) & 1;
+  if (CH == 4) return (n >> 1) & 3;
+  if (CH == 8) return n & 7;
+  return n & 15;
+}
+
+template <int N> __device__ __forceinline__ void waitVmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+constexpr int cmin(int a, int b) { return a < b ? a : b; }
+
+template <class T, int CIN, int COUT, int KS, int MT, int WAVES, int NS, bool RESIDENT>
+__global__ void __launch_bounds__(64 * WAVES)
+convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
+           const int32_t* __restrict__ nbr, const T* __restrict__ zeros, int kVol, int64_t inRows, int64_t outRows,
+           int relu, int tileBlocks) {
+  constexpr int THREADS = 64 * WAVES;
+  constexpr int CS = CIN / KS;                                 // input channels per step (a tap takes KS steps)
+  constexpr int CH = CS * static_cast<int>(sizeof(T)) / 16;    // 16-byte chunks of a row staged per step
+  constexpr int RPI = 64 / CH;                                 // rows one gather instruction covers
+  constexpr int WM = 16 * MT, TM = WAVES * WM;
+  constexpr int GL = WM / RPI;                                 // gather instructions per tap
+  static_assert(WM % RPI == 0 && WM <= 64, "wavefront tile");
+  constexpr int NT = COUT / 16;
+  constexpr int KSTEP = CIN >= 32 ? 32 : 16;
+  constexpr int KK = CS / KSTEP;
+  constexpr int WCH = CS * COUT / 8;                           // 16-byte chunks of one step's weights
+  static_assert(WCH % 64 == 0 && KK >= 1, "weights per step");
+  constexpr int WL = RESIDENT ? 0 : (WCH + THREADS - 1) / THREADS;
+  constexpr int NWB = 3, NI = 4;
+  constexpr int SLOTS = WM * CH;                               // 16-byte slots per stage
+  constexpr int OCH = COUT * static_cast<int>(sizeof(T)) / 16; // chunks per output row
+  constexpr bool LDS_EPILOGUE = WM * OCH <= NS * SLOTS;
+  // Issue order inside step a: indices of step a+NS+3, weights of step a+2, rows of step a+NS.  X = loads that
+  // may still be in flight when the step ends, behind the rows and the weights of step a+1.
+  constexpr int PER_STEP = 1 + WL + GL;
+  constexpr int X_ROWS = (NS - 1) * PER_STEP;
+  constexpr int X_WEIGHTS = RESIDENT ? 63 : GL + PER_STEP;
+  constexpr int X_INDEX = WL + GL + 2 * PER_STEP;
+  constexpr int X = cmin(cmin(X_ROWS, X_WEIGHTS), cmin(X_INDEX, 63));
+  using F = typename Frag<CIN>::type;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15, kgrp = lane >> 4;
+  const int steps = kVol * KS;                                 // step s = tap s / KS, channel part s % KS
+  const int wChunks = (RESIDENT ? steps : NWB) * WCH;
+  u32x4* wLds = reinterpret_cast<u32x4*>(smem);
+  int32_t* idxLds = reinterpret_cast<int32_t*>(smem + static_cast<size_t>(wChunks) * 16) + wave * NI * 64;
+  u32x4* stage = reinterpret_cast<u32x4*>(smem + static_cast<size_t>(wChunks) * 16 + WAVES * NI * 256) + wave * NS * SLOTS;
+
+  if (RESIDENT) {
+    const u32x4* src = reinterpret_cast<const u32x4*>(wf);
+    for (int e = tid; e < steps * WCH; e += THREADS) wLds[e] = src[e];
+    __syncthreads();
+  }
+
+  const int perXcd = (tileBlocks + 7) / 8;
+  const int xcd = blockIdx.x & 7;
+  for (int local = blockIdx.x >> 3; local < perXcd; local += gridDim.x >> 3) {
+    const int tile = xcd * perXcd + local;
+    if (tile >= tileBlocks) break;                     // workgroup-uniform
+    const int64_t row0 = static_cast<int64_t>(tile) * TM + wave * WM;
+
+    auto issueIndex = [&](int t) __attribute__((always_inline)) {
+      int64_t row = row0 + lane;
+      if (row >= outRows) row = outRows - 1;
+      __builtin_amdgcn_global_load_lds(nbr + static_cast<int64_t>(t / KS) * outRows + row, idxLds + (t & (NI - 1)) * 64, 4, 0, 0);
+    };
+    auto issueWeights = [&](int t) __attribute__((always_inline)) {
+      const u32x4* wk = reinterpret_cast<const u32x4*>(wf) + static_cast<size_t>(t) * WCH;
+      const int buf = t % NWB;
+#pragma unroll
+      for (int q = 0; q < WL; ++q) {
+        const int base = (q * THREADS + wave * 64) % WCH;  // wavefronts past the slice repeat a part of it: same bytes
+        __builtin_amdgcn_global_load_lds(wk + base + lane, wLds + buf * WCH + base, 16, 0, 0);
+      }
+    };
+    auto issueRows = [&](int t, int slot) __attribute__((always_inline)) {
+      const int32_t* ix = idxLds + (t & (NI - 1)) * 64;
+      int32_t src[GL];
+#pragma unroll
+      for (int j = 0; j < GL; ++j) src[j] = ix[j * RPI + lane / CH];
+#pragma unroll
+      for (int j = 0; j < GL; ++j) {
+        const int n = j * RPI + lane / CH;
+        const int c = (lane % CH) ^ stageSwizzle<CH>(n);
+        const bool ok = src[j] >= 0 && src[j] < inRows && row0 + n < outRows;
+        const T* p = (ok ? in + static_cast<size_t>(src[j]) * CIN + (t % KS) * CS : zeros) + c * 8;
+        // (a half-precision pointer here makes the host pass drop the kernel's launch stub without a diagnostic)
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(p), stage + slot * SLOTS + j * 64, 16, 0, 0);
+      }
+    };
+
+    // prologue: indices and rows of the first NS steps, the first two weight slices, indices of the next three steps
+    for (int t = 0; t < NS && t < steps; ++t) issueIndex(t);
+    if (!RESIDENT) {
+      issueWeights(0);
+      if (steps > 1) issueWeights(1);
+    }
+    waitVmcnt<0>();
+    for (int t = 0; t < NS && t < steps; ++t) issueRows(t, t);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // index slots are reused by the next three steps
+    for (int t = NS; t < NS + 3 && t < steps; ++t) issueIndex(t);
+    waitVmcnt<0>();
+    if (!RESIDENT) __syncthreads();
+
+    float4v acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int n = 0; n < NT; ++n) acc[m][n] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    int slot = 0, wbuf = 0;
+    for (int a = 0; a < steps; ++a) {
+      const bool steady = a + NS + 3 < steps;
+      if (steady) issueIndex(a + NS + 3);
+      if (!RESIDENT && a + 2 < steps) issueWeights(a + 2);
+      F rows[MT][KK];
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const int n = m * 16 + r16;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          if constexpr (CIN >= 32) {
+            rows[m][kk] = stage[slot * SLOTS + n * CH + ((kk * 4 + kgrp) ^ stageSwizzle<CH>(n))];
+          } else {
+            const u32x2* s2 = reinterpret_cast<const u32x2*>(stage + slot * SLOTS + n * CH + ((kgrp >> 1) ^ stageSwizzle<CH>(n)));
+            rows[m][kk] = s2[kgrp & 1];
+          }
+        }
+      }
+      if (a + NS < steps) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot has been read before it is refilled
+        issueRows(a + NS, slot);
+      }
+      const F* wTap = reinterpret_cast<const F*>(wLds + (RESIDENT ? a : wbuf) * WCH);
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+          const F wfrag = wTap[(kk * NT + n) * 64 + lane];
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            if constexpr (CIN >= 32) {
+              acc[m][n] = Mfma<T>::k32(wfrag, rows[m][kk], acc[m][n]);
+            } else {
+              acc[m][n] = Mfma<T>::k16(wfrag, rows[m][kk], acc[m][n]);
+            }
+          }
+        }
+      }
+      if (steady) {
+        waitVmcnt<X>();
+      } else {
+        // the last steps issue fewer loads: count what may stay in flight behind the ones step a+1 needs
+        auto issued = [&](int s_) __attribute__((always_inline)) {
+          return (s_ + NS + 3 < steps ? 1 : 0) + (s_ + 2 < steps ? WL : 0) + (s_ + NS < steps ? GL : 0);
+        };
+        int allowed = 0;
+        if (a + 1 < steps) {
+          allowed = 63;
+          if (a + 1 >= NS) {  // rows of step a+1 left in step a+1-NS, the last loads of that step
+            int r = 0;
+            for (int s_ = a + 2 - NS; s_ <= a; ++s_) r += issued(s_);
+            allowed = r < allowed ? r : allowed;
+          }
+          if (!RESIDENT && a >= 1) {  // weights of step a+1 left in step a-1, before that step's rows
+            const int w = (a - 1 + NS < steps ? GL : 0) + issued(a);
+            allowed = w < allowed ? w : allowed;
+          }
+          if (a + 1 + NS < steps && a >= 2) {  // indices of step a+1+NS left first in step a-2
+            const int i_ = issued(a - 2) - 1 + issued(a - 1) + issued(a);
+            allowed = i_ < allowed ? i_ : allowed;
+          }
+        }
+        if (allowed >= X) waitVmcnt<X>();
+        else if (allowed >= PER_STEP - 1) waitVmcnt<cmin(PER_STEP - 1, 63)>();
+        else if (allowed >= GL) waitVmcnt<cmin(GL, 63)>();
+        else waitVmcnt<0>();
+      }
+      if (!RESIDENT) __syncthreads();
+      slot = slot + 1 == NS ? 0 : slot + 1;
+      wbuf = wbuf + 1 == NWB ? 0 : wbuf + 1;
+    }
+
+    // epilogue: bias, ReLU, rounding; rows leave through the stage area as contiguous lines
+    if constexpr (LDS_EPILOGUE) {
+      unsigned char* sb = reinterpret_cast<unsigned char*>(stage);
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const int n_ = m * 16 + r16;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+          const int col = n * 16 + kgrp * 4;
+          float v[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v[j] = acc[m][n][j] + (bias ? bias[col + j] : 0.f);
+            if (relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
+          }
+          T packed[4] = {static_cast<T>(v[0]), static_cast<T>(v[1]), static_cast<T>(v[2]), static_cast<T>(v[3])};
+          const int oc = (col >> 3) ^ stageSwizzle<OCH>(n_);
+          *reinterpret_cast<u32x2*>(sb + (n_ * OCH + oc) * 16 + (kgrp & 1) * 8) = __builtin_bit_cast(u32x2, packed);
+        }
+      }
+      constexpr int ORPI = 64 / OCH;
+#pragma unroll
+      for (int j = 0; j < WM / ORPI; ++j) {
+        const int n_ = j * ORPI + lane / OCH;
+        const int c = lane % OCH;
+        const u32x4 v = stage[n_ * OCH + (c ^ stageSwizzle<OCH>(n_))];
+        const int64_t row = row0 + n_;
+        if (row < outRows) *reinterpret_cast<u32x4*>(out + static_cast<size_t>(row) * COUT + c * 8) = v;
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the stage is free again before the next tile's rows land
+    } else {
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const int64_t row = row0 + m * 16 + r16;
+        if (row >= outRows) continue;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+          const int col = n * 16 + kgrp * 4;
+          float v[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v[j] = acc[m][n][j] + (bias ? bias[col + j] : 0.f);
+            if (relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
+          }
+          T packed[4] = {static_cast<T>(v[0]), static_cast<T>(v[1]), static_cast<T>(v[2]), static_cast<T>(v[3])};
+          *reinterpret_cast<u32x2*>(out + static_cast<size_t>(row) * COUT + col) = __builtin_bit_cast(u32x2, packed);
+        }
+      }
+    }
+  }
+}
+
 constexpr size_t kLdsLimit = 160 * 1024;
 
 template <int CIN, int COUT>
@@ -604,10 +871,66 @@ int32_t launchMfmaResident(const ConvArgs& a, hipStream_t stream) {
   return D3D_OK;
 }
 
+template <class T, int CIN, int COUT, int KS, int MT, int WAVES, int NS, bool RESIDENT>
+int32_t launchStagedCfg(const ConvArgs& a, hipStream_t stream) {
+  constexpr int CH = CIN / KS * static_cast<int>(sizeof(T)) / 16;
+  constexpr int WM = 16 * MT, TM = WM * WAVES;
+  constexpr int WCH = CIN / KS * COUT / 8;
+  const size_t lds = static_cast<size_t>(RESIDENT ? a.kVol * KS : 3) * WCH * 16 + static_cast<size_t>(WAVES) * 4 * 256 +
+                     static_cast<size_t>(WAVES) * NS * WM * CH * 16;
+  if (lds > kLdsLimit) return D3D_ERR_UNSUPPORTED;  // the caller falls back
+  static size_t granted = 64 * 1024;
+  const int32_t rc = grantLds(&convStaged<T, CIN, COUT, KS, MT, WAVES, NS, RESIDENT>, lds, &granted);
+  if (rc != D3D_OK) return rc;
+  const int tiles = static_cast<int>((a.outRows + TM - 1) / TM);
+  int blocks = (tiles + 7) / 8 * 8;
+  if (RESIDENT) {  // persistent workgroups share one weight load
+    int perCu = static_cast<int>(kLdsLimit / lds);
+    if (perCu > 2) perCu = 2;
+    if (blocks > 256 * perCu) blocks = 256 * perCu;
+  }
+  hipLaunchKernelGGL((convStaged<T, CIN, COUT, KS, MT, WAVES, NS, RESIDENT>), dim3(static_cast<unsigned>(blocks)),
+                     dim3(64 * WAVES), lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
+                     static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, static_cast<const T*>(a.zeros), a.kVol,
+                     a.inRows, a.outRows, a.relu, tiles);
+  return D3D_OK;
+}
+
+// Configuration of the staged kernel: rows per wavefront (16*MT), wavefronts, stage depth, weights resident or
+// streamed.  `a.staged` (tests, tuning) = MT | WAVES << 8 | NS << 16 | resident << 24; 0 = choose here.
+template <class T, int CIN, int COUT>
+int32_t launchStaged(const ConvArgs& a, hipStream_t stream) {
+  constexpr bool SMALL = CIN * COUT <= 1024;  // 27 taps of weights fit beside the stages
+  constexpr int KS = CIN > 64 ? CIN / 64 : 1; // at most 64 channels are staged per step
+  int cfg = a.staged;
+  if (cfg == 0) {  // measured on the layers of a VoxelNet backbone (120k voxels)
+    if (CIN == 16) return D3D_ERR_UNSUPPORTED;              // 32-byte rows: the register-gather kernels are faster
+    if (CIN * COUT >= 16384) cfg = 2 | 8 << 8 | 3 << 16;
+    else if (CIN * COUT >= 8192 || CIN * COUT == 2048) cfg = 2 | 8 << 8 | 2 << 16;
+    else cfg = 4 | 8 << 8 | 2 << 16;
+  }
+  switch (cfg) {
+    case 4 | 8 << 8 | 2 << 16: if constexpr (CIN * COUT < 8192) return launchStagedCfg<T, CIN, COUT, KS, 4, 8, 2, false>(a, stream); break;
+    case 2 | 8 << 8 | 3 << 16: return launchStagedCfg<T, CIN, COUT, KS, 2, 8, 3, false>(a, stream);
+    case 2 | 8 << 8 | 2 << 16: return launchStagedCfg<T, CIN, COUT, KS, 2, 8, 2, false>(a, stream);
+    case 4 | 4 << 8 | 2 << 16: return launchStagedCfg<T, CIN, COUT, KS, 4, 4, 2, false>(a, stream);
+    case 4 | 4 << 8 | 3 << 16: return launchStagedCfg<T, CIN, COUT, KS, 4, 4, 3, false>(a, stream);
+    case 4 | 8 << 8 | 3 << 16 | 1 << 24: if constexpr (SMALL) return launchStagedCfg<T, CIN, COUT, KS, 4, 8, 3, true>(a, stream); break;
+    case 2 | 8 << 8 | 3 << 16 | 1 << 24: if constexpr (SMALL) return launchStagedCfg<T, CIN, COUT, KS, 2, 8, 3, true>(a, stream); break;
+  }
+  return D3D_ERR_UNSUPPORTED;
+}
+
 // Small layers keep every tap's weights in LDS (convMfmaResident).  Large layers stream one tap's weights at a
 // time through LDS for 8 (or 4) wavefronts; more rows per wavefront (MT) amortise that stream.
 template <class T, int CIN, int COUT>
 int32_t launchMfmaOne(const ConvArgs& a, hipStream_t stream) {
+  if constexpr (CIN * COUT >= 512) {
+    if (a.staged >= 0) {
+      const int32_t rc = launchStaged<T, CIN, COUT>(a, stream);
+      if (rc != D3D_ERR_UNSUPPORTED) return rc;
+    }
+  }
   const size_t allTaps = static_cast<size_t>(a.kVol) * CIN * COUT * sizeof(T);
   if (allTaps <= 56 * 1024 && a.kVol <= 128 && allTaps + static_cast<size_t>(16) * a.kVol * 16 * 4 <= kLdsLimit)
     return launchMfmaResident<T, CIN, COUT>(a, stream);

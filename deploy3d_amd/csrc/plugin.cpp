@@ -456,6 +456,17 @@ int tileRowsOverride() {
   return v | ((w && std::atoi(w) == 4) ? (1 << 30) : 0);
 }
 
+// Tuning / test hook: D3D_CONV_STAGED = "off" keeps the register-gather kernels; "MT,WAVES,NS[,1]" picks a
+// configuration of the staged kernel (trailing 1 = weights resident in LDS); unset = heuristic.
+int stagedOverride() {
+  const char* e = std::getenv("D3D_CONV_STAGED");
+  if (!e || !*e) return 0;
+  if (std::strcmp(e, "off") == 0) return -1;
+  int mt = 0, waves = 0, ns = 0, res = 0;
+  if (std::sscanf(e, "%d,%d,%d,%d", &mt, &waves, &ns, &res) < 3) return 0;
+  return mt | waves << 8 | ns << 16 | (res ? 1 << 24 : 0);
+}
+
 // --- SPConvMM ----------------------------------------------------------------
 // Attribute layout: SPConvMMPluginParam + fp32 payload, trt/spconv/mm_trt.cu:27-37, :61-68.
 constexpr uint32_t kExtMagic = 0x58443344u;  // "D3DX"
@@ -658,6 +669,7 @@ struct MMPlugin final : d3d_plugin {
     a.relu = relu ? 1 : 0;
     a.zeros = zeros;
     a.tileRows = tileRowsOverride();
+    a.staged = stagedOverride();
     return launchConv(a, stream);
   }
 };

@@ -107,7 +107,19 @@ def test_kernel_shapes(engine, ksize, padding):
 def test_mfma_tile_sizes(engine, monkeypatch, tile_rows, cin, cout):
     """Every workgroup tile height of the MFMA kernel (the launcher normally picks one from the row count)."""
     monkeypatch.setenv("D3D_CONV_TILE_ROWS", str(tile_rows))
+    monkeypatch.setenv("D3D_CONV_STAGED", "off")
     run_case(3001, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, "float16", True, relu=True)
+
+
+@pytest.mark.parametrize("cfg", ["off", "4,8,2", "2,8,3", "2,8,2", "4,4,2", "4,4,3", "4,8,3,1", "2,8,3,1"])
+@pytest.mark.parametrize("cin,cout", [(16, 32), (32, 32), (32, 64), (64, 64), (64, 128), (128, 128), (128, 16)])
+def test_staged_configurations(engine, monkeypatch, cfg, cin, cout):
+    """Every configuration of the LDS-staged MFMA kernel (rows per wavefront, wavefronts, stage depth, resident
+    weights), and the register-gather kernels behind "off"; a configuration a layer does not support falls back."""
+    monkeypatch.setenv("D3D_CONV_STAGED", cfg)
+    run_case(3001, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, "float16", True, relu=True)
+    if cfg in ("4,8,2", "2,8,3", "off"):
+        run_case(2100, (10, 36, 30), (3, 1, 1), (2, 1, 1), (0, 0, 0), cin, cout, "bfloat16", False)
 
 
 def test_no_bias_no_relu(engine):
