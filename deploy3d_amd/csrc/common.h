@@ -69,10 +69,11 @@ size_t rulebookWorkspaceBytes(const RbGeom& g, int64_t cap, bool subM, bool grid
 
 // Builds one rulebook on `stream`.  coors [cap, nd+1]; numActIn device int32.
 // index [3, rowLen] with rowLen = kVol * (cap + 128).  outCoors / numActOut are
-// null for SubM.  Returns a D3D status.
+// null for SubM.  When nbrOut is given (16-byte aligned, [kVol, nbrRows]) the pairs are also written in
+// output-major form, nbrOut[tap][output row] = input row, -1 elsewhere.  Returns a D3D status.
 int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const int32_t* numActIn, int64_t cap,
                        int32_t maxNumActOut, int32_t* index, int32_t* numIndex, int32_t* outCoors, int32_t* numActOut,
-                       void* workspace, size_t workspaceBytes, hipStream_t stream);
+                       void* workspace, size_t workspaceBytes, int32_t* nbrOut, int64_t nbrRows, hipStream_t stream);
 
 // Out-major neighbour table of one rulebook: nbr[tap, row] = gathered input row
 // or -1, rows = maxNumActOut.  Built from the index tensor (optionally with the

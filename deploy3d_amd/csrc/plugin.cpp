@@ -176,6 +176,36 @@ void noteRulebookWritten(const void* index) {
   ++e.generation;
 }
 
+// The rulebook operator can write the forward table itself while it compacts the pairs.  This reserves the
+// buffer of the entry (null if that fails or D3D_RULEBOOK_NBR=0 asks for the derived form)...
+int32_t* reserveForwardTable(const void* index, int kVol, int64_t outRows) {
+  const char* env = std::getenv("D3D_RULEBOOK_NBR");
+  if ((env && env[0] == '0') || outRows <= 0) return nullptr;
+  std::lock_guard<std::mutex> lock(g_cacheMutex);
+  NbrTable& t = g_cache[index].forward;
+  const size_t bytes = static_cast<size_t>(kVol) * static_cast<size_t>(outRows) * sizeof(int32_t);
+  if (!t.buf || t.buf->bytes < bytes) {
+    auto nb = std::make_shared<DeviceBuffer>();
+    if (nb->reserve(bytes) != D3D_OK) return nullptr;
+    t.buf = nb;
+    t.built = false;
+  }
+  return static_cast<int32_t*>(t.buf->ptr);
+}
+
+// ... and this records, with the new generation, that the table in it is current.
+void noteForwardTableWritten(const void* index, int kVol, int64_t outRows, int64_t rowLen, const void* numIndex) {
+  std::lock_guard<std::mutex> lock(g_cacheMutex);
+  NbrEntry& e = g_cache[index];
+  NbrTable& t = e.forward;
+  t.built = true;
+  t.builtGeneration = e.generation;
+  t.kVol = kVol;
+  t.outRows = outRows;
+  t.rowLen = rowLen;
+  t.numIndex = numIndex;
+}
+
 int32_t neighbourTable(const int32_t* index, int64_t rowLen, const int32_t* numIndex, bool inverse, int kVol,
                        int64_t outRows, hipStream_t stream, std::shared_ptr<DeviceBuffer>* out) {
   std::lock_guard<std::mutex> lock(g_cacheMutex);
@@ -419,12 +449,17 @@ struct IdxPlugin final : d3d_plugin {
       }
     }
     const RbGeom g = geometry(grid);
+    int32_t* nbr = reserveForwardTable(outputs[0], kVol(), maxNumActOut);
     int32_t rc = launchRulebook(g, subM, static_cast<const int32_t*>(inputs[0]),
                                 static_cast<const int32_t*>(inputs[1]), cap, maxNumActOut,
                                 static_cast<int32_t*>(outputs[0]), static_cast<int32_t*>(outputs[1]),
                                 subM ? nullptr : static_cast<int32_t*>(outputs[2]),
-                                subM ? nullptr : static_cast<int32_t*>(outputs[3]), workspace, workspaceBytes, stream);
-    if (rc == D3D_OK) noteRulebookWritten(outputs[0]);
+                                subM ? nullptr : static_cast<int32_t*>(outputs[3]), workspace, workspaceBytes, nbr,
+                                maxNumActOut, stream);
+    if (rc == D3D_OK) {
+      noteRulebookWritten(outputs[0]);
+      if (nbr) noteForwardTableWritten(outputs[0], kVol(), maxNumActOut, rowLen, outputs[1]);
+    }
     return rc;
   }
 };

@@ -453,7 +453,7 @@ __global__ void __launch_bounds__(kRbThreads)
 rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int kVol,
           const uint32_t* __restrict__ staging, const uint32_t* __restrict__ cnt, uint32_t nBlocks,
           const uint32_t* __restrict__ totals, int32_t* __restrict__ gather, int32_t* __restrict__ scatter,
-          int32_t* __restrict__ tapRow, int32_t* numIndex) {
+          int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* __restrict__ nbr, int64_t nbrRows) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int tap = blockIdx.y;
   const uint32_t b = blockIdx.x;
@@ -487,8 +487,19 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
       scatter[at] = static_cast<int32_t>(v[j]);
       tapRow[at] = tap;
       ++at;
+      // the same pair in output-major form, for the convolution: nbr[tap][output row] = input row
+      if (nbr && v[j] < static_cast<uint64_t>(nbrRows)) nbr[static_cast<int64_t>(tap) * nbrRows + v[j]] = static_cast<int32_t>(first + j);
     }
   }
+}
+
+__global__ void __launch_bounds__(kRbThreads) rbFillMinusOne(int32_t* p, int64_t n) {  // p is 16-byte aligned
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  uint4* p4 = reinterpret_cast<uint4*>(p);
+  const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
+  for (int64_t i = tid; i < n / 4; i += stride) p4[i] = ones;
+  if (tid < (n & 3)) p[(n & ~static_cast<int64_t>(3)) + tid] = -1;
 }
 
 // ===========================================================================
@@ -1079,7 +1090,7 @@ RbWorkspace planRulebookWorkspace(const RbGeom& g, int64_t cap, bool subM, size_
 
 int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const int32_t* numActIn, int64_t cap,
                        int32_t maxNumActOut, int32_t* index, int32_t* numIndex, int32_t* outCoors, int32_t* numActOut,
-                       void* workspace, size_t workspaceBytes, hipStream_t stream) {
+                       void* workspace, size_t workspaceBytes, int32_t* nbrOut, int64_t nbrRows, hipStream_t stream) {
   if (!coors || !numActIn || !index || !numIndex || (!subM && (!outCoors || !numActOut))) {
     setError("rulebook: null tensor pointer");
     return D3D_ERR_BAD_ARG;
@@ -1197,8 +1208,11 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
                          cnt, w.nBlocks, totals);
     }
   }
+  if (nbrOut && nbrRows > 0)
+    hipLaunchKernelGGL(rbFillMinusOne, fillGrid(static_cast<int64_t>(g.kVol) * nbrRows / 4 + 1), block, 0, stream, nbrOut,
+                       static_cast<int64_t>(g.kVol) * nbrRows);
   hipLaunchKernelGGL(rbCompact, perTap, block, 0, stream, numActIn, cap, w.pitch, g.kVol, staging, cnt, w.nBlocks,
-                     totals, index, index + rowLen, index + 2 * rowLen, numIndex);
+                     totals, index, index + rowLen, index + 2 * rowLen, numIndex, nbrRows > 0 ? nbrOut : nullptr, nbrRows);
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;
 }
