@@ -73,6 +73,8 @@ def main():
     ap.add_argument("--voxels", type=int, default=120000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager enqueues instead of HIP-graph replays")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="enqueue rulebooks and convolutions on one stream instead of two")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="end with ONE device-to-device copy of this many MiB: the dispatch of known size that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this script")
@@ -96,7 +98,7 @@ def main():
     n = len(cfg["coords"])
     counts = layers.measure_output_counts(specs, cfg["coords"], cfg["grid"])
     caps = layers.plan_capacities(specs, n, counts)
-    net = layers.SparseBackbone(specs, weights, caps)
+    net = layers.SparseBackbone(specs, weights, caps, overlap=not args.no_overlap)
     x = layers.make_input(cfg["coords"], cfg["feats"], cfg["grid"])
 
     stream = torch.cuda.Stream()
@@ -142,7 +144,7 @@ def main():
                 y = net.forward(x)
             stream.synchronize()
             ms = (time.perf_counter() - t0) * 1e3 / args.steps
-            mode = "eager"
+            mode = "eager" + ("" if args.no_overlap else ", rulebooks beside convolutions on a second stream")
         else:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
@@ -156,7 +158,7 @@ def main():
                 graph.replay()
             torch.cuda.synchronize()
             ms = (time.perf_counter() - t0) * 1e3 / args.steps
-            mode = "hip-graph replay"
+            mode = "hip-graph replay" + ("" if args.no_overlap else ", rulebooks beside convolutions on a second stream")
         same = bool(torch.equal(y.feats, ref_out))
         if args.pmc_copy_mib:
             src = torch.ones(args.pmc_copy_mib << 20, dtype=torch.uint8, device="cuda")

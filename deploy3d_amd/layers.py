@@ -96,15 +96,35 @@ class SparseConvLayer:
 
 
 class SparseBackbone:
-    """A chain (or small DAG, via ``src``) of SparseConvLayers sharing rulebooks by indice key."""
+    """A chain (or small DAG, via ``src``) of SparseConvLayers sharing rulebooks by indice key.
 
-    def __init__(self, layers, weights, capacities, dtype=torch.float16, device="cuda"):
+    Rulebooks depend on coordinates only, convolutions on features and on their rulebook.  With ``overlap``
+    (the default) the rulebooks are enqueued on a second HIP stream and every convolution waits for the event
+    of its own rulebook, so the latency-bound index kernels of later stages run beside the MFMA kernels of
+    earlier ones.  The side stream forks from and joins into the caller's current stream, so a forward pass can
+    still be captured into one HIP graph (it then holds two parallel branches).  (A third stream for the SubM
+    rulebooks, which only depend on the strided ones, made hipStreamEndCapture crash in the runtime; the
+    single side stream is what is supported.)
+    """
+
+    def __init__(self, layers, weights, capacities, dtype=torch.float16, device="cuda", overlap=True):
         self.specs = layers
         self.layers = [SparseConvLayer(s, w, b, cap, dtype=dtype, device=device)
                        for s, (w, b), cap in zip(layers, weights, capacities)]
+        self.overlap = overlap
+        self._side = None
 
     def forward(self, x):
+        main = side = None
+        if self.overlap:
+            if self._side is None:
+                self._side = torch.cuda.Stream()
+            main, side = torch.cuda.current_stream(), self._side
+            fork = torch.cuda.Event()
+            fork.record(main)
+            side.wait_event(fork)
         rulebooks = {}
+        pending = {}
         outs = {"input": x}
         cur = x
         for spec, lyr in zip(self.specs, self.layers):
@@ -116,6 +136,14 @@ class SparseBackbone:
                 inp = SparseTensor(a.feats + b.feats, a.coors, a.num_act, a.grid, a.batch)
             else:
                 inp = outs[src]
+            key = spec["key"]
+            if side is not None and key not in rulebooks:
+                with torch.cuda.stream(side):
+                    rulebooks[key] = lyr.build_rulebook(inp)
+                    pending[key] = torch.cuda.Event()
+                    pending[key].record(side)
+            if key in pending:
+                main.wait_event(pending.pop(key))
             cur = lyr.forward(inp, rulebooks)
             outs[spec["name"]] = cur
         self.rulebooks = rulebooks
