@@ -997,10 +997,43 @@ int32_t launchNarrow(const ConvArgs& a, hipStream_t stream) {
 
 bool isMfmaChannels(int c) { return c == 16 || c == 32 || c == 64 || c == 128; }
 
+// rows of `cin` 2-byte channels widened to `cinPad` (a multiple of 8) with zeros, so that a narrow first layer
+// (5 input channels, say) can run on the MFMA path
+__global__ void __launch_bounds__(256)
+padRows(const uint16_t* __restrict__ in, int64_t rows, int cin, int cinPad, uint16_t* __restrict__ out) {
+  const int chunks = cinPad / 8;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; e < rows * chunks; e += stride) {
+    const int64_t row = e / chunks;
+    const int c0 = static_cast<int>(e % chunks) * 8;
+    uint16_t v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = c0 + j < cin ? in[row * cin + c0 + j] : static_cast<uint16_t>(0);
+    *reinterpret_cast<u32x4*>(out + row * cinPad + c0) = __builtin_bit_cast(u32x4, v);
+  }
+}
+
 }  // namespace
 
 bool convUsesMfma(int32_t dtype, int cin, int cout) {
   return (dtype == D3D_HALF || dtype == D3D_BF16) && isMfmaChannels(cin) && isMfmaChannels(cout);
+}
+
+int paddedMfmaChannels(int32_t dtype, int cin, int cout) {
+  if ((dtype != D3D_HALF && dtype != D3D_BF16) || !isMfmaChannels(cout) || cin < 1 || cin > 128) return cin;
+  int c = 16;
+  while (c < cin) c *= 2;
+  return c;
+}
+
+int32_t launchPadRows(const void* in, int64_t rows, int cin, int cinPad, void* out, hipStream_t stream) {
+  if (rows <= 0) return D3D_OK;
+  int64_t blocks = (rows * (cinPad / 8) + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(padRows, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                     static_cast<const uint16_t*>(in), rows, cin, cinPad, static_cast<uint16_t*>(out));
+  D3D_HIP_CHECK(hipGetLastError());
+  return D3D_OK;
 }
 
 int32_t launchBuildNeighbours(const int32_t* index, int64_t rowLen, const int32_t* numIndex, bool inverse, int kVol,

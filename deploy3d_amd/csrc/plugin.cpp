@@ -509,6 +509,7 @@ constexpr size_t kMMHeader = 19;
 
 struct MMDeviceWeights {
   int32_t dtype = -1;
+  int cinMfma = 0;  // input channels of the packed MFMA weights (cin widened with zero rows), 0 = no MFMA copy
   DeviceBuffer f32, mfma, bias;
 };
 
@@ -520,6 +521,7 @@ struct MMPlugin final : d3d_plugin {
   std::shared_ptr<MMDeviceWeights> dev;        // shared by clones (mm_trt.cu:43-45, :75-79)
   std::shared_ptr<std::mutex> devMutex;
   std::shared_ptr<DeviceBuffer> lastTable;     // keeps the table of the last enqueue alive
+  std::shared_ptr<DeviceBuffer> widened;       // input rows widened to the MFMA channel count (narrow layers)
 
   static int32_t parse(const void* data, size_t len, MMPlugin** out) {
     if (!data || len < kMMHeader) {
@@ -573,7 +575,12 @@ struct MMPlugin final : d3d_plugin {
     return D3D_OK;
   }
 
-  d3d_plugin* clone() const override { return new MMPlugin(*this); }
+  d3d_plugin* clone() const override {
+    auto* c = new MMPlugin(*this);  // weights are shared (mm_trt.cu:75-79); per-enqueue buffers are not
+    c->lastTable.reset();
+    c->widened.reset();
+    return c;
+  }
   int32_t numOutputs() const override { return 1; }
   int32_t outputDims(int32_t idx, const d3d_tensor_desc*, int32_t, d3d_tensor_desc* out) const override {
     if (idx != 0 || !out) return D3D_ERR_BAD_ARG;
@@ -612,17 +619,21 @@ struct MMPlugin final : d3d_plugin {
     std::memcpy(w.data(), blob.data() + weightOffset, nW * 4);
     if (withBias) std::memcpy(b.data(), blob.data() + weightOffset + nW * 4, static_cast<size_t>(cout) * 4);
     std::vector<uint16_t> packed;
+    int cinMfma = 0;
     if (dtype == D3D_HALF || dtype == D3D_BF16) {
       const bool half = dtype == D3D_HALF;
       auto rnd = [&](float v, uint16_t* bits) {
         *bits = half ? floatToHalfBits(v) : floatToBf16Bits(v);
         return half ? halfBitsToFloat(*bits) : bf16BitsToFloat(*bits);
       };
-      const bool mfma = convUsesMfma(dtype, cin, cout);
-      if (mfma) packed.resize(nW);
+      const int cinP = paddedMfmaChannels(dtype, cin, cout);
+      const bool mfma = convUsesMfma(dtype, cinP, cout);
+      if (mfma) packed.assign(static_cast<size_t>(kernelVol) * cinP * cout, 0);
+      cinMfma = mfma ? cinP : 0;
       // fragment-major copy for the MFMA kernel: Wf[tap][kk][n][lane][j] = W[tap][kk*KS + (lane/16)*KG + j][n*16 + lane%16]
-      // with KS = 32 (16 when cin == 16) and KG = KS/4, so one wavefront load fetches one whole operand fragment
-      const int ks = cin >= 32 ? 32 : 16, kg = ks / 4, nt = cout / 16, kkN = cin / ks;
+      // with KS = 32 (16 when cin == 16) and KG = KS/4, so one wavefront load fetches one whole operand fragment;
+      // rows past cin (a narrow layer widened to 16 channels) stay zero
+      const int ks = cinP >= 32 ? 32 : 16, kg = ks / 4, nt = cout / 16, kkN = cinP / ks;
       for (int k = 0; k < kernelVol; ++k)
         for (int ci = 0; ci < cin; ++ci)
           for (int co = 0; co < cout; ++co) {
@@ -643,7 +654,7 @@ struct MMPlugin final : d3d_plugin {
     int32_t rc = dev->f32.upload(w.data(), nW * 4);
     if (rc != D3D_OK) return rc;
     if (!packed.empty()) {
-      rc = dev->mfma.upload(packed.data(), nW * 2);
+      rc = dev->mfma.upload(packed.data(), packed.size() * 2);
       if (rc != D3D_OK) return rc;
     }
     if (withBias) {
@@ -654,6 +665,7 @@ struct MMPlugin final : d3d_plugin {
       setError("SPConvMM: could not allocate the zero row");
       return D3D_ERR_DEVICE;
     }
+    dev->cinMfma = cinMfma;
     dev->dtype = dtype;
     return D3D_OK;
   }
@@ -696,6 +708,16 @@ struct MMPlugin final : d3d_plugin {
     a.inRows = inDesc[0].dims[0];
     a.outRows = outRows;
     a.in = inputs[0];
+    if (dev->cinMfma > cin && (reinterpret_cast<uintptr_t>(outputs[0]) & 15) == 0 &&
+        std::getenv("D3D_CONV_NO_PAD") == nullptr) {  // narrow layer: widen the rows, then MFMA
+      if (!widened) widened = std::make_shared<DeviceBuffer>();
+      rc = widened->reserve(static_cast<size_t>(a.inRows > 0 ? a.inRows : 1) * dev->cinMfma * 2);
+      if (rc != D3D_OK) return rc;
+      rc = launchPadRows(inputs[0], a.inRows, cin, dev->cinMfma, widened->ptr, stream);
+      if (rc != D3D_OK) return rc;
+      a.in = widened->ptr;
+      a.cin = dev->cinMfma;
+    }
     a.out = outputs[0];
     a.weightsF32 = static_cast<const float*>(dev->f32.ptr);
     a.weightsMfma = dev->mfma.ptr;

@@ -122,6 +122,16 @@ def test_staged_configurations(engine, monkeypatch, cfg, cin, cout):
         run_case(2100, (10, 36, 30), (3, 1, 1), (2, 1, 1), (0, 0, 0), cin, cout, "bfloat16", False)
 
 
+@pytest.mark.parametrize("cin,cout", [(5, 16), (3, 32), (20, 32), (40, 64), (100, 128)])
+@pytest.mark.parametrize("padded", [True, False])
+def test_widened_input_channels(engine, monkeypatch, cin, cout, padded):
+    """A layer whose output channels fit the MFMA path but whose input channels do not runs on rows widened with
+    zero channels (weights widened with zero rows); D3D_CONV_NO_PAD keeps it on the narrow-channel kernel."""
+    if not padded:
+        monkeypatch.setenv("D3D_CONV_NO_PAD", "1")
+    run_case(3000, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, "float16", True, relu=True, cap_extra=77)
+
+
 def test_no_bias_no_relu(engine):
     run_case(2500, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), 32, 32, "float16", True, with_bias=False)
 
