@@ -579,19 +579,47 @@ bmReset(uint4* records16, int64_t nRecords, int32_t* index, int64_t nIndex, uint
   if (tid == 0) *numIndex = 0;
 }
 
+// Lanes of a 16-lane row that target the same record merge their bits before the atomic: inputs usually arrive
+// in brick order, so neighbouring lanes hit the same record and device-wide atomic throughput (the bound of the
+// marking passes) is spent on one operation per run instead of one per voxel.  `rec` = kNone for lanes with
+// nothing to mark.  Bits only accumulate with OR, so merging any equal-record lanes is valid; the last lane of
+// each run of equal records issues the atomic.
+__device__ __forceinline__ void orRuns(BmRecord* records, uint32_t rec, unsigned long long bits) {
+  uint32_t lo = static_cast<uint32_t>(bits), hi = static_cast<uint32_t>(bits >> 32);
+  const int key = static_cast<int>(rec);
+#define D3D_ROW_SHR_STEP(N)                                                                        \
+  {                                                                                                \
+    const int k2 = __builtin_amdgcn_update_dpp(-2, key, 0x110 + N, 0xF, 0xF, false);               \
+    const uint32_t lo2 = __builtin_amdgcn_update_dpp(0, static_cast<int>(lo), 0x110 + N, 0xF, 0xF, false); \
+    const uint32_t hi2 = __builtin_amdgcn_update_dpp(0, static_cast<int>(hi), 0x110 + N, 0xF, 0xF, false); \
+    if (k2 == key) {                                                                               \
+      lo |= lo2;                                                                                   \
+      hi |= hi2;                                                                                   \
+    }                                                                                              \
+  }
+  D3D_ROW_SHR_STEP(1)
+  D3D_ROW_SHR_STEP(2)
+  D3D_ROW_SHR_STEP(4)
+  D3D_ROW_SHR_STEP(8)
+#undef D3D_ROW_SHR_STEP
+  const int next = __builtin_amdgcn_update_dpp(-2, key, 0x101, 0xF, 0xF, false);  // row_shl:1 = the next lane's record
+  if (rec != kNone && next != key && (lo | hi))
+    atomicOr(&records[rec].bits, (static_cast<unsigned long long>(hi) << 32) | lo);
+}
+
 // SubM: mark the input voxels.
 __global__ void __launch_bounds__(kRbThreads)
 bmMarkInputs(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
              BmRecord* records) {
   const int n = liveCount(numActIn, cap);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  int c[5];
-  loadCoord(coors, g.nd, i, c);
-  if (!coordInGrid(g, c)) return;
-  uint32_t rec, bit;
-  bmLocate(m, c, &rec, &bit);
-  atomicOr(&records[rec].bits, 1ull << bit);
+  uint32_t rec = kNone, bit = 0;
+  if (i < n) {
+    int c[5];
+    loadCoord(coors, g.nd, i, c);
+    if (coordInGrid(g, c)) bmLocate(m, c, &rec, &bit);
+  }
+  orRuns(records, rec, 1ull << bit);  // every lane takes part in the cross-lane merge
 }
 
 // Strided / transposed: mark every candidate output (reference: convGeometryKernel, index.cu:86-102).
@@ -858,32 +886,30 @@ __device__ __forceinline__ uint32_t nearMembers(const BlockMap& m, const NearBas
   return present;
 }
 
-// Strided / transposed: one thread marks all candidate outputs of one input,
-// one atomicOr per brick of its group (and none where a read shows the bits set).
+// Strided / transposed: one thread marks all candidate outputs of one input: per brick of its group one
+// atomicOr for each run of neighbouring lanes that target the same brick.
 __global__ void __launch_bounds__(kRbThreads)
 bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
            BmRecord* records) {
   __shared__ unsigned long long masks[kNearGroup][kRbThreads];
   const int n = liveCount(numActIn, cap);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kRbThreads + threadIdx.x;
-  if (i >= n) return;
-  int c[5];
-  loadCoord(coors, g.nd, i, c);
+  const bool live = i < n;
+  int c[5] = {0, 0, 0, 0, 0};
+  if (live) loadCoord(coors, g.nd, i, c);
   const NearBase b = nearBase(g, m, c);
   uint32_t rec[kNearGroup];
-  const uint32_t present = nearMembers(m, b, rec);
-  unsigned long long have[kNearGroup];
-#pragma unroll
-  for (int e = 0; e < kNearGroup; ++e) have[e] = __builtin_nontemporal_load(&records[rec[e]].bits);
+  const uint32_t present = live ? nearMembers(m, b, rec) : (nearMembers(m, b, rec), 0u);
 #pragma unroll
   for (int e = 0; e < kNearGroup; ++e) masks[e][threadIdx.x] = 0ull;
-  nearForEachTap(g, m, c, b, [&](int, bool ok, int member, uint32_t bit) {
-    if (ok) masks[member][threadIdx.x] |= 1ull << bit;
-  });
+  if (live)
+    nearForEachTap(g, m, c, b, [&](int, bool ok, int member, uint32_t bit) {
+      if (ok) masks[member][threadIdx.x] |= 1ull << bit;
+    });
 #pragma unroll
   for (int e = 0; e < kNearGroup; ++e) {
     const unsigned long long want = masks[e][threadIdx.x];
-    if (((present >> e) & 1u) && (have[e] & want) != want) atomicOr(&records[rec[e]].bits, want);
+    orRuns(records, ((present >> e) & 1u) && want ? rec[e] : kNone, want);
   }
 }
 
