@@ -493,14 +493,6 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
   }
 }
 
-__global__ void __launch_bounds__(kRbThreads) rbFillMinusOne(int32_t* p, int64_t n) {  // p is 16-byte aligned
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  uint4* p4 = reinterpret_cast<uint4*>(p);
-  const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
-  for (int64_t i = tid; i < n / 4; i += stride) p4[i] = ones;
-  if (tid < (n & 3)) p[(n & ~static_cast<int64_t>(3)) + tid] = -1;
-}
 
 // ===========================================================================
 // Block-map path.  When the grid is small enough to afford 16 bytes per 64
@@ -558,25 +550,36 @@ __device__ __forceinline__ uint32_t bmRank(const BmRecord& r, uint32_t bit) {
 }
 
 // reset for the block-map path: records = 0, index tensor = -1, counters = 0
+// -1 over p[0..n) by the threads tid, tid+stride, ...: 16-byte stores over the aligned body
+__device__ __forceinline__ void fillMinusOneRange(int32_t* p, int64_t n, int64_t tid, int64_t stride) {
+  if (!p || n <= 0) return;
+  const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
+  const uintptr_t base = reinterpret_cast<uintptr_t>(p);
+  int64_t head = ((16 - (base & 15)) & 15) >> 2;
+  if (head > n) head = n;
+  const int64_t body16 = (n - head) >> 2;
+  uint4* body = reinterpret_cast<uint4*>(p + head);
+  for (int64_t i = tid; i < body16; i += stride) body[i] = ones;
+  const int64_t tailStart = head + (body16 << 2);
+  if (tid < head) p[tid] = -1;
+  if (tid < n - tailStart) p[tailStart + tid] = -1;
+}
+
 __global__ void __launch_bounds__(kRbThreads)
 bmReset(uint4* records16, int64_t nRecords, int32_t* index, int64_t nIndex, uint32_t* counters, int64_t nCounters,
         int32_t* numIndex) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const uint4 zero = make_uint4(0, 0, 0, 0);
-  const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
   for (int64_t i = tid; i < nRecords; i += stride) records16[i] = zero;
-  const uintptr_t base = reinterpret_cast<uintptr_t>(index);
-  int64_t head = ((16 - (base & 15)) & 15) >> 2;
-  if (head > nIndex) head = nIndex;
-  const int64_t body16 = (nIndex - head) >> 2;
-  uint4* body = reinterpret_cast<uint4*>(index + head);
-  for (int64_t i = tid; i < body16; i += stride) body[i] = ones;
-  const int64_t tailStart = head + (body16 << 2);
-  if (tid < head) index[tid] = -1;
-  if (tid < nIndex - tailStart) index[tailStart + tid] = -1;
+  fillMinusOneRange(index, nIndex, tid, stride);  // index == nullptr: a later pass fills it
   for (int64_t q = tid; q < nCounters; q += stride) counters[q] = 0;
   if (tid == 0) *numIndex = 0;
+}
+
+__global__ void __launch_bounds__(kRbThreads) rbFillMinusOne(int32_t* p, int64_t n) {
+  fillMinusOneRange(p, n, static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x,
+                    static_cast<int64_t>(gridDim.x) * blockDim.x);
 }
 
 // Lanes of a 16-lane row that target the same record merge their bits before the atomic: inputs usually arrive
@@ -920,12 +923,26 @@ __global__ void __launch_bounds__(kRbThreads)
 bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
             int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ perm,
             const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
-            uint32_t* cnt, uint32_t nBlocks, uint32_t* totals) {
+            uint32_t* cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
+            int64_t nFillB, uint32_t fillBlocks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char nearSmem[];
   uint4* group = reinterpret_cast<uint4*>(nearSmem);                                   // [8][kRbThreads] records
   uint32_t* ldsCnt = reinterpret_cast<uint32_t*>(group + kNearGroup * kRbThreads);    // [kVol]
+  // Every fourth workgroup is a fill workgroup: the -1 fill of the index tensor and of the neighbour table is
+  // bandwidth-bound, this pass latency-bound, and neither depends on the other, so they share one launch.
+  const uint32_t quad = blockIdx.x >> 2, part = blockIdx.x & 3;
+  if (part == 3) {
+    if (quad < fillBlocks) {
+      const int64_t tid = static_cast<int64_t>(quad) * kRbThreads + threadIdx.x;
+      const int64_t stride = static_cast<int64_t>(fillBlocks) * kRbThreads;
+      fillMinusOneRange(fillA, nFillA, tid, stride);
+      fillMinusOneRange(fillB, nFillB, tid, stride);
+    }
+    return;
+  }
+  const uint32_t probeBlock = quad * 3 + part;
   const int n = liveCount(numActIn, cap);
-  const int64_t i0 = static_cast<int64_t>(blockIdx.x) * kRbThreads;
+  const int64_t i0 = static_cast<int64_t>(probeBlock) * kRbThreads;
   if (i0 >= n) return;  // workgroup-uniform
   for (int t = threadIdx.x; t < g.kVol; t += blockDim.x) ldsCnt[t] = 0;
   const bool shuffled = SUBM && *permShuffled != 0;  // rows are not already in rank order
@@ -962,7 +979,7 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
     if ((threadIdx.x & 63) == 0 && hit) atomicAdd(&ldsCnt[tap], static_cast<uint32_t>(__popcll(hit)));
   });
   __syncthreads();
-  const uint32_t chunk = blockIdx.x / kRbItems;
+  const uint32_t chunk = probeBlock / kRbItems;
   for (int t = threadIdx.x; t < g.kVol; t += blockDim.x) {
     const uint32_t v = ldsCnt[t];
     if (v) {
@@ -1167,6 +1184,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     return dim3(static_cast<unsigned>(blocks < 1 ? 1 : blocks));
   };
 
+  bool nbrFilled = false;
   if (w.blockMap) {
     uint64_t nRecords64;
     const BlockMap m = makeBlockMap(g, &nRecords64);
@@ -1177,9 +1195,10 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     uint32_t* permShuffled = totals + 2 * g.kVol;
     const bool near = nearEligible(g, m);
     const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
-    hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + nIndex / 4 + 1), block, 0, stream,
-                       reinterpret_cast<uint4*>(records), static_cast<int64_t>(w.nRecords), index, nIndex, cnt,
-                       static_cast<int64_t>(g.kVol) * w.nBlocks + 2 * g.kVol + 1, numIndex);
+    hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + (near ? 0 : nIndex / 4) + 1), block, 0,
+                       stream, reinterpret_cast<uint4*>(records), static_cast<int64_t>(w.nRecords),
+                       near ? nullptr : index, nIndex, cnt, static_cast<int64_t>(g.kVol) * w.nBlocks + 2 * g.kVol + 1,
+                       numIndex);
     if (subM) {
       hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
     } else if (near) {
@@ -1196,13 +1215,21 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     if (subM)
       hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, perm,
                          permShuffled);
-    if (near) {
+    if (near) {  // probe workgroups interleaved 3:1 with fill workgroups (index tensor, neighbour table)
+      const uint32_t probeBlocks = perInput.x;
+      const uint32_t quads = (probeBlocks + 2) / 3;
+      const dim3 fused(quads * 4);
+      int32_t* fillB = (nbrOut && nbrRows > 0) ? nbrOut : nullptr;
+      const int64_t nFillB = fillB ? static_cast<int64_t>(g.kVol) * nbrRows : 0;
+      nbrFilled = true;
       if (subM) {
-        hipLaunchKernelGGL(bmProbeNear<true>, perInput, block, nearLds, stream, g, m, coors, numActIn, cap,
-                           w.pitch, records, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
+        hipLaunchKernelGGL(bmProbeNear<true>, fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,
+                           records, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
+                           fillB, nFillB, quads);
       } else {
-        hipLaunchKernelGGL(bmProbeNear<false>, perInput, block, nearLds, stream, g, m, coors, numActIn, cap,
-                           w.pitch, records, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
+        hipLaunchKernelGGL(bmProbeNear<false>, fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,
+                           records, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
+                           fillB, nFillB, quads);
       }
     } else if (subM) {
       hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, perm,
@@ -1234,7 +1261,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
                          cnt, w.nBlocks, totals);
     }
   }
-  if (nbrOut && nbrRows > 0)
+  if (nbrOut && nbrRows > 0 && !nbrFilled)
     hipLaunchKernelGGL(rbFillMinusOne, fillGrid(static_cast<int64_t>(g.kVol) * nbrRows / 4 + 1), block, 0, stream, nbrOut,
                        static_cast<int64_t>(g.kVol) * nbrRows);
   hipLaunchKernelGGL(rbCompact, perTap, block, 0, stream, numActIn, cap, w.pitch, g.kVol, staging, cnt, w.nBlocks,
