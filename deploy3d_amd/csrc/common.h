@@ -108,6 +108,6 @@ bool convUsesMfma(int32_t dtype, int cin, int cout);
 // Input-channel count the MFMA path would run a layer at (the next of 16/32/64/128 for 2-byte types when the
 // output channels qualify), else cin itself; and the kernel that widens rows to it with zero channels.
 int paddedMfmaChannels(int32_t dtype, int cin, int cout);
-int32_t launchPadRows(const void* in, int64_t rows, int cin, int cinPad, void* out, hipStream_t stream);
+int32_t launchPadRows(const void* in, int64_t rows, int inBytes, int outBytes, void* out, hipStream_t stream);
 
 }  // namespace d3d

@@ -24,6 +24,7 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef int32_t int4v __attribute__((ext_vector_type(4)));
 
 constexpr int kConvThreads = 256;
 constexpr int kTileRows = 64;
@@ -184,6 +185,7 @@ convNarrow(const T* __restrict__ in, T* __restrict__ out, const float* __restric
 // ---------------------------------------------------------------------------
 template <class T> struct Mfma;
 template <> struct Mfma<_Float16> {
+  using Acc = float4v;
   __device__ static float4v k32(const u32x4& a, const u32x4& b, const float4v& c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0,
                                                   0);
@@ -194,6 +196,7 @@ template <> struct Mfma<_Float16> {
   }
 };
 template <> struct Mfma<__bf16> {
+  using Acc = float4v;
   __device__ static float4v k32(const u32x4& a, const u32x4& b, const float4v& c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                    0, 0);
@@ -201,6 +204,17 @@ template <> struct Mfma<__bf16> {
   __device__ static float4v k16(const u32x2& a, const u32x2& b, const float4v& c) {
     return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4v, a), __builtin_bit_cast(short4v, b), c,
                                                      0, 0, 0);
+  }
+};
+
+// int8 operands, int32 accumulators: 16x16x64 takes 16 bytes per lane, 16x16x32 takes 8.
+template <> struct Mfma<int8_t> {
+  using Acc = int4v;
+  __device__ static int4v k32(const u32x4& a, const u32x4& b, const int4v& c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(int4v, a), __builtin_bit_cast(int4v, b), c, 0, 0, 0);
+  }
+  __device__ static int4v k16(const u32x2& a, const u32x2& b, const int4v& c) {
+    return __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b), c, 0, 0, 0);
   }
 };
 
@@ -584,25 +598,28 @@ constexpr int cmin(int a, int b) { return a < b ? a : b; }
 template <class T, int CIN, int COUT, int KS, int MT, int WAVES, int NS, bool RESIDENT>
 __global__ void __launch_bounds__(64 * WAVES)
 convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
-           const int32_t* __restrict__ nbr, const T* __restrict__ zeros, int kVol, int64_t inRows, int64_t outRows,
+           const float* __restrict__ requantM, const int32_t* __restrict__ nbr, const T* __restrict__ zeros, int kVol, int64_t inRows, int64_t outRows,
            int relu, int tileBlocks) {
   constexpr int THREADS = 64 * WAVES;
+  constexpr int ES = static_cast<int>(sizeof(T));              // 2: fp16 / bf16, 1: int8
+  constexpr int EPC = 16 / ES;                                 // elements per 16-byte chunk
   constexpr int CS = CIN / KS;                                 // input channels per step (a tap takes KS steps)
-  constexpr int CH = CS * static_cast<int>(sizeof(T)) / 16;    // 16-byte chunks of a row staged per step
+  constexpr int CH = CS * ES / 16;                             // 16-byte chunks of a row staged per step
+  constexpr bool WIDE = CS * ES >= 64;                         // 16-byte operand fragments (else 8-byte)
   constexpr int RPI = 64 / CH;                                 // rows one gather instruction covers
   constexpr int WM = 16 * MT, TM = WAVES * WM;
   constexpr int GL = WM / RPI;                                 // gather instructions per tap
   static_assert(WM % RPI == 0 && WM <= 64, "wavefront tile");
   constexpr int NT = COUT / 16;
-  constexpr int KSTEP = CIN >= 32 ? 32 : 16;
+  constexpr int KSTEP = (WIDE ? 64 : 32) / ES;                 // channels one MFMA contracts
   constexpr int KK = CS / KSTEP;
-  constexpr int WCH = CS * COUT / 8;                           // 16-byte chunks of one step's weights
+  constexpr int WCH = CS * COUT * ES / 16;                     // 16-byte chunks of one step's weights
   static_assert(WCH % 64 == 0 && KK >= 1, "weights per step");
   constexpr int WL = RESIDENT ? 0 : (WCH + THREADS - 1) / THREADS;
   constexpr int NWB = 3, NI = 4;
   constexpr int SLOTS = WM * CH;                               // 16-byte slots per stage
-  constexpr int OCH = COUT * static_cast<int>(sizeof(T)) / 16; // chunks per output row
-  constexpr bool LDS_EPILOGUE = WM * OCH <= NS * SLOTS;
+  constexpr int OCH = COUT * ES / 16;                          // chunks per output row
+  constexpr bool LDS_EPILOGUE = ES == 2 && WM * OCH <= NS * SLOTS;
   // Issue order inside step a: indices of step a+NS+3, weights of step a+2, rows of step a+NS.  X = loads that
   // may still be in flight when the step ends, behind the rows and the weights of step a+1.
   constexpr int PER_STEP = 1 + WL + GL;
@@ -610,7 +627,8 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
   constexpr int X_WEIGHTS = RESIDENT ? 63 : GL + PER_STEP;
   constexpr int X_INDEX = WL + GL + 2 * PER_STEP;
   constexpr int X = cmin(cmin(X_ROWS, X_WEIGHTS), cmin(X_INDEX, 63));
-  using F = typename Frag<CIN>::type;
+  using F = typename Frag<WIDE ? 32 : 16>::type;
+  using Acc = typename Mfma<T>::Acc;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
@@ -660,7 +678,7 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
         const int n = j * RPI + lane / CH;
         const int c = (lane % CH) ^ stageSwizzle<CH>(n);
         const bool ok = src[j] >= 0 && src[j] < inRows && row0 + n < outRows;
-        const T* p = (ok ? in + static_cast<size_t>(src[j]) * CIN + (t % KS) * CS : zeros) + c * 8;
+        const T* p = (ok ? in + static_cast<size_t>(src[j]) * CIN + (t % KS) * CS : zeros) + c * EPC;
         // (a half-precision pointer here makes the host pass drop the kernel's launch stub without a diagnostic)
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(p), stage + slot * SLOTS + j * 64, 16, 0, 0);
       }
@@ -679,11 +697,11 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
     waitVmcnt<0>();
     if (!RESIDENT) __syncthreads();
 
-    float4v acc[MT][NT];
+    Acc acc[MT][NT];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int n = 0; n < NT; ++n) acc[m][n] = float4v{0.f, 0.f, 0.f, 0.f};
+      for (int n = 0; n < NT; ++n) acc[m][n] = Acc{0, 0, 0, 0};
 
     int slot = 0, wbuf = 0;
     for (int a = 0; a < steps; ++a) {
@@ -696,7 +714,7 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
         const int n = m * 16 + r16;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
-          if constexpr (CIN >= 32) {
+          if constexpr (WIDE) {
             rows[m][kk] = stage[slot * SLOTS + n * CH + ((kk * 4 + kgrp) ^ stageSwizzle<CH>(n))];
           } else {
             const u32x2* s2 = reinterpret_cast<const u32x2*>(stage + slot * SLOTS + n * CH + ((kgrp >> 1) ^ stageSwizzle<CH>(n)));
@@ -716,7 +734,7 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
           const F wfrag = wTap[(kk * NT + n) * 64 + lane];
 #pragma unroll
           for (int m = 0; m < MT; ++m) {
-            if constexpr (CIN >= 32) {
+            if constexpr (WIDE) {
               acc[m][n] = Mfma<T>::k32(wfrag, rows[m][kk], acc[m][n]);
             } else {
               acc[m][n] = Mfma<T>::k16(wfrag, rows[m][kk], acc[m][n]);
@@ -788,6 +806,27 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
         if (row < outRows) *reinterpret_cast<u32x4*>(out + static_cast<size_t>(row) * COUT + c * 8) = v;
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the stage is free again before the next tile's rows land
+    } else if constexpr (ES == 1) {
+      // int8: t = float(acc) * m[c]; t += bq[c]; round to nearest even; clamp (lo = 0 with the fused ReLU)
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const int64_t row = row0 + m * 16 + r16;
+        if (row >= outRows) continue;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+          const int col = n * 16 + kgrp * 4;
+          uint32_t packed = 0;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            float t = static_cast<float>(acc[m][n][j]) * requantM[col + j];
+            t = t + (bias ? bias[col + j] : 0.f);
+            float q = __builtin_rintf(t);
+            q = __builtin_fminf(127.f, __builtin_fmaxf(relu ? 0.f : -128.f, q));
+            packed |= (static_cast<uint32_t>(static_cast<int>(q)) & 0xFFu) << (8 * j);
+          }
+          *reinterpret_cast<uint32_t*>(out + static_cast<size_t>(row) * COUT + col) = packed;
+        }
+      }
     } else {
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
@@ -875,7 +914,7 @@ template <class T, int CIN, int COUT, int KS, int MT, int WAVES, int NS, bool RE
 int32_t launchStagedCfg(const ConvArgs& a, hipStream_t stream) {
   constexpr int CH = CIN / KS * static_cast<int>(sizeof(T)) / 16;
   constexpr int WM = 16 * MT, TM = WM * WAVES;
-  constexpr int WCH = CIN / KS * COUT / 8;
+  constexpr int WCH = CIN / KS * COUT * static_cast<int>(sizeof(T)) / 16;
   const size_t lds = static_cast<size_t>(RESIDENT ? a.kVol * KS : 3) * WCH * 16 + static_cast<size_t>(WAVES) * 4 * 256 +
                      static_cast<size_t>(WAVES) * NS * WM * CH * 16;
   if (lds > kLdsLimit) return D3D_ERR_UNSUPPORTED;  // the caller falls back
@@ -891,8 +930,8 @@ int32_t launchStagedCfg(const ConvArgs& a, hipStream_t stream) {
   }
   hipLaunchKernelGGL((convStaged<T, CIN, COUT, KS, MT, WAVES, NS, RESIDENT>), dim3(static_cast<unsigned>(blocks)),
                      dim3(64 * WAVES), lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
-                     static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, static_cast<const T*>(a.zeros), a.kVol,
-                     a.inRows, a.outRows, a.relu, tiles);
+                     static_cast<const T*>(a.weightsMfma), a.bias, a.requantM, a.nbr, static_cast<const T*>(a.zeros),
+                     a.kVol, a.inRows, a.outRows, a.relu, tiles);
   return D3D_OK;
 }
 
@@ -901,10 +940,11 @@ int32_t launchStagedCfg(const ConvArgs& a, hipStream_t stream) {
 template <class T, int CIN, int COUT>
 int32_t launchStaged(const ConvArgs& a, hipStream_t stream) {
   constexpr bool SMALL = CIN * COUT <= 1024;  // 27 taps of weights fit beside the stages
-  constexpr int KS = CIN > 64 ? CIN / 64 : 1; // at most 64 channels are staged per step
+  constexpr int ROWB = CIN * static_cast<int>(sizeof(T));
+  constexpr int KS = ROWB > 128 ? ROWB / 128 : 1;  // at most 128 bytes of a row are staged per step
   int cfg = a.staged;
   if (cfg == 0) {  // measured on the layers of a VoxelNet backbone (120k voxels)
-    if (CIN == 16) return D3D_ERR_UNSUPPORTED;              // 32-byte rows: the register-gather kernels are faster
+    if (CIN == 16 && sizeof(T) == 2) return D3D_ERR_UNSUPPORTED;  // 32-byte rows: the register-gather kernels are faster
     if (CIN * COUT >= 16384) cfg = 2 | 8 << 8 | 3 << 16;
     else if (CIN * COUT >= 8192 || CIN * COUT == 2048) cfg = 2 | 8 << 8 | 2 << 16;
     else cfg = 4 | 8 << 8 | 2 << 16;
@@ -997,41 +1037,70 @@ int32_t launchNarrow(const ConvArgs& a, hipStream_t stream) {
 
 bool isMfmaChannels(int c) { return c == 16 || c == 32 || c == 64 || c == 128; }
 
-// rows of `cin` 2-byte channels widened to `cinPad` (a multiple of 8) with zeros, so that a narrow first layer
+// rows of `inBytes` bytes widened to `outBytes` (a multiple of 16) with zeros, so that a narrow first layer
 // (5 input channels, say) can run on the MFMA path
 __global__ void __launch_bounds__(256)
-padRows(const uint16_t* __restrict__ in, int64_t rows, int cin, int cinPad, uint16_t* __restrict__ out) {
-  const int chunks = cinPad / 8;
+padRows(const uint8_t* __restrict__ in, int64_t rows, int inBytes, int outBytes, uint8_t* __restrict__ out) {
+  const int chunks = outBytes / 16;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; e < rows * chunks; e += stride) {
     const int64_t row = e / chunks;
-    const int c0 = static_cast<int>(e % chunks) * 8;
-    uint16_t v[8];
+    const int c0 = static_cast<int>(e % chunks) * 16;
+    uint8_t v[16];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = c0 + j < cin ? in[row * cin + c0 + j] : static_cast<uint16_t>(0);
-    *reinterpret_cast<u32x4*>(out + row * cinPad + c0) = __builtin_bit_cast(u32x4, v);
+    for (int j = 0; j < 16; ++j) v[j] = c0 + j < inBytes ? in[row * inBytes + c0 + j] : static_cast<uint8_t>(0);
+    *reinterpret_cast<u32x4*>(out + row * outBytes + c0) = __builtin_bit_cast(u32x4, v);
   }
+}
+
+template <int CIN>
+int32_t launchInt8Cout(const ConvArgs& a, hipStream_t stream) {
+  switch (a.cout) {
+    case 16: if constexpr (CIN * 16 >= 1024) return launchStaged<int8_t, CIN, 16>(a, stream); break;
+    case 32: return launchStaged<int8_t, CIN, 32>(a, stream);
+    case 64: return launchStaged<int8_t, CIN, 64>(a, stream);
+    case 128: return launchStaged<int8_t, CIN, 128>(a, stream);
+  }
+  return D3D_ERR_UNSUPPORTED;
+}
+
+int32_t launchInt8(const ConvArgs& a, hipStream_t stream) {
+  switch (a.cin) {
+    case 32: return launchInt8Cout<32>(a, stream);
+    case 64: return launchInt8Cout<64>(a, stream);
+    case 128: return launchInt8Cout<128>(a, stream);
+  }
+  return D3D_ERR_UNSUPPORTED;
 }
 
 }  // namespace
 
 bool convUsesMfma(int32_t dtype, int cin, int cout) {
+  if (dtype == D3D_INT8) return (cin == 32 || cin == 64 || cin == 128) && isMfmaChannels(cout) && cin * cout >= 1024;
   return (dtype == D3D_HALF || dtype == D3D_BF16) && isMfmaChannels(cin) && isMfmaChannels(cout);
 }
 
 int paddedMfmaChannels(int32_t dtype, int cin, int cout) {
-  if ((dtype != D3D_HALF && dtype != D3D_BF16) || !isMfmaChannels(cout) || cin < 1 || cin > 128) return cin;
-  int c = 16;
-  while (c < cin) c *= 2;
-  return c;
+  if (!isMfmaChannels(cout) || cin < 1 || cin > 128) return cin;
+  if (dtype == D3D_HALF || dtype == D3D_BF16) {
+    int c = 16;
+    while (c < cin) c *= 2;
+    return c;
+  }
+  if (dtype == D3D_INT8) {  // the int8 MFMA contracts at least 32 channels; a step's weights fill at least 1 KiB
+    int c = 32;
+    while (c < cin || c * cout < 1024) c *= 2;
+    return c <= 128 ? c : cin;
+  }
+  return cin;
 }
 
-int32_t launchPadRows(const void* in, int64_t rows, int cin, int cinPad, void* out, hipStream_t stream) {
+int32_t launchPadRows(const void* in, int64_t rows, int inBytes, int outBytes, void* out, hipStream_t stream) {
   if (rows <= 0) return D3D_OK;
-  int64_t blocks = (rows * (cinPad / 8) + 255) / 256;
+  int64_t blocks = (rows * (outBytes / 16) + 255) / 256;
   if (blocks > 4096) blocks = 4096;
   hipLaunchKernelGGL(padRows, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
-                     static_cast<const uint16_t*>(in), rows, cin, cinPad, static_cast<uint16_t*>(out));
+                     static_cast<const uint8_t*>(in), rows, inBytes, outBytes, static_cast<uint8_t*>(out));
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;
 }
@@ -1058,7 +1127,15 @@ int32_t launchConv(const ConvArgs& a, hipStream_t stream) {
   if (a.outRows <= 0) return D3D_OK;
   int32_t rc = D3D_ERR_UNSUPPORTED;
   const bool aligned = ((reinterpret_cast<uintptr_t>(a.in) | reinterpret_cast<uintptr_t>(a.out)) & 15) == 0;
-  if (convUsesMfma(a.dtype, a.cin, a.cout) && aligned && a.weightsMfma && a.zeros) {
+  if (a.dtype == D3D_INT8) {
+    if (!convUsesMfma(a.dtype, a.cin, a.cout) || !aligned || !a.weightsMfma || !a.zeros || !a.requantM) {
+      setError("conv: int8 needs 32/64/128 (widened) input channels, 16/32/64/128 output channels, 16-byte aligned "
+               "tensors and requantize scales");
+      return D3D_ERR_UNSUPPORTED;
+    }
+    rc = launchInt8(a, stream);
+    if (rc == D3D_ERR_UNSUPPORTED) setError("conv: int8 layer does not fit the staged kernel (kernel volume %d)", a.kVol);
+  } else if (convUsesMfma(a.dtype, a.cin, a.cout) && aligned && a.weightsMfma && a.zeros) {
     rc = a.dtype == D3D_HALF ? launchMfma<_Float16>(a, stream) : launchMfma<__bf16>(a, stream);
   } else {
     switch (a.dtype) {

@@ -510,7 +510,7 @@ constexpr size_t kMMHeader = 19;
 struct MMDeviceWeights {
   int32_t dtype = -1;
   int cinMfma = 0;  // input channels of the packed MFMA weights (cin widened with zero rows), 0 = no MFMA copy
-  DeviceBuffer f32, mfma, bias;
+  DeviceBuffer f32, mfma, bias, requantM;  // int8: bias holds bias / s_out, requantM holds s_in * s_w[c] / s_out
 };
 
 struct MMPlugin final : d3d_plugin {
@@ -594,7 +594,7 @@ struct MMPlugin final : d3d_plugin {
   int32_t outputDtype(int32_t, const int32_t* inTypes, int32_t nbIn) const override {
     return (inTypes && nbIn > 0) ? inTypes[0] : D3D_ERR_BAD_ARG;  // mm_trt.cu:104-106
   }
-  static bool featureType(int32_t t) { return t == D3D_HALF || t == D3D_FLOAT || t == D3D_BF16; }
+  static bool featureType(int32_t t) { return t == D3D_HALF || t == D3D_FLOAT || t == D3D_BF16 || t == D3D_INT8; }
   int32_t supportsFormat(int32_t pos, const d3d_tensor_desc* io, int32_t nbIn, int32_t nbOut) const override {
     if (!io || pos < 0 || pos >= nbIn + nbOut || io[pos].format != D3D_LINEAR) return 0;
     if (pos == 0) return featureType(io[0].dtype);
@@ -614,6 +614,7 @@ struct MMPlugin final : d3d_plugin {
     }
     std::lock_guard<std::mutex> lock(*devMutex);
     if (dev->dtype == dtype) return D3D_OK;
+    if (dtype == D3D_INT8) return configureInt8();
     const size_t nW = static_cast<size_t>(kernelVol) * cin * cout;
     std::vector<float> w(nW), b(withBias ? cout : 0);
     std::memcpy(w.data(), blob.data() + weightOffset, nW * 4);
@@ -670,6 +671,61 @@ struct MMPlugin final : d3d_plugin {
     return D3D_OK;
   }
 
+  // int8 (no counterpart in the reference): symmetric per-output-channel weights, s_w[c] = max|W[:,:,c]| / 127,
+  // q = clamp(rint(w / s_w)); the epilogue computes clamp(rint(float(acc) * m[c] + bq[c])) with
+  // m[c] = float(s_in * s_w[c] / s_out) and bq[c] = float(bias[c] / s_out), all three quotients in double.
+  int32_t configureInt8() {
+    if (!(actScaleIn > 0.f) || !(actScaleOut > 0.f)) {
+      setError("SPConvMM: int8 needs positive activation scales in the extension record");
+      return D3D_ERR_UNSUPPORTED;
+    }
+    const int cinP = paddedMfmaChannels(D3D_INT8, cin, cout);
+    if (!convUsesMfma(D3D_INT8, cinP, cout)) {
+      setError("SPConvMM: int8 is implemented for up to 128 input channels and 16/32/64/128 output channels");
+      return D3D_ERR_UNSUPPORTED;
+    }
+    const size_t nW = static_cast<size_t>(kernelVol) * cin * cout;
+    std::vector<float> w(nW), b(cout, 0.f);
+    std::memcpy(w.data(), blob.data() + weightOffset, nW * 4);
+    if (withBias) std::memcpy(b.data(), blob.data() + weightOffset + nW * 4, static_cast<size_t>(cout) * 4);
+    std::vector<double> sw(cout, 0.0);
+    for (size_t i = 0; i < nW; ++i) {
+      const double v = std::fabs(static_cast<double>(w[i]));
+      if (v > sw[i % cout]) sw[i % cout] = v;
+    }
+    std::vector<float> m(cout), bq(cout);
+    for (int c = 0; c < cout; ++c) {
+      sw[c] = sw[c] / 127.0;
+      if (sw[c] == 0.0) sw[c] = 1.0;
+      m[c] = static_cast<float>(static_cast<double>(actScaleIn) * sw[c] / static_cast<double>(actScaleOut));
+      bq[c] = static_cast<float>(static_cast<double>(b[c]) / static_cast<double>(actScaleOut));
+    }
+    // fragment-major: Wf[tap][kk][n][lane][j] = q[tap][kk*KS + (lane/16)*KG + j][n*16 + lane%16], KS = 64 (32), KG = KS/4
+    const int ks = cinP >= 64 ? 64 : 32, kg = ks / 4, nt = cout / 16, kkN = cinP / ks;
+    std::vector<int8_t> packed(static_cast<size_t>(kernelVol) * cinP * cout, 0);
+    for (int k = 0; k < kernelVol; ++k)
+      for (int ci = 0; ci < cin; ++ci)
+        for (int co = 0; co < cout; ++co) {
+          const size_t src = (static_cast<size_t>(k) * cin + ci) * cout + co;
+          double q = std::nearbyint(static_cast<double>(w[src]) / sw[co]);
+          q = q > 127.0 ? 127.0 : (q < -127.0 ? -127.0 : q);
+          const int kk = ci / ks, within = ci % ks, lane = (within / kg) * 16 + co % 16, j = within % kg;
+          const size_t dst = (((static_cast<size_t>(k) * kkN + kk) * nt + co / 16) * 64 + lane) * kg + j;
+          packed[dst] = static_cast<int8_t>(q);
+        }
+    int32_t rc = dev->mfma.upload(packed.data(), packed.size());
+    if (rc == D3D_OK) rc = dev->requantM.upload(m.data(), m.size() * 4);
+    if (rc == D3D_OK) rc = dev->bias.upload(bq.data(), bq.size() * 4);
+    if (rc != D3D_OK) return rc;
+    if (!zeroRow()) {
+      setError("SPConvMM: could not allocate the zero row");
+      return D3D_ERR_DEVICE;
+    }
+    dev->cinMfma = cinP;
+    dev->dtype = D3D_INT8;
+    return D3D_OK;
+  }
+
   size_t workspaceSize(const d3d_tensor_desc*, int32_t) const override { return 0; }  // mm_trt.cu:143-148
 
   int32_t enqueue(const d3d_tensor_desc* inDesc, const d3d_tensor_desc* outDesc, const void* const* inputs,
@@ -708,12 +764,13 @@ struct MMPlugin final : d3d_plugin {
     a.inRows = inDesc[0].dims[0];
     a.outRows = outRows;
     a.in = inputs[0];
-    if (dev->cinMfma > cin && (reinterpret_cast<uintptr_t>(outputs[0]) & 15) == 0 &&
-        std::getenv("D3D_CONV_NO_PAD") == nullptr) {  // narrow layer: widen the rows, then MFMA
+    if (dev->cinMfma > cin && (dtype == D3D_INT8 || ((reinterpret_cast<uintptr_t>(outputs[0]) & 15) == 0 &&
+                                                     std::getenv("D3D_CONV_NO_PAD") == nullptr))) {  // narrow layer: widen the rows, then MFMA
       if (!widened) widened = std::make_shared<DeviceBuffer>();
-      rc = widened->reserve(static_cast<size_t>(a.inRows > 0 ? a.inRows : 1) * dev->cinMfma * 2);
+      const int es = dtypeBytes(dtype);
+      rc = widened->reserve(static_cast<size_t>(a.inRows > 0 ? a.inRows : 1) * dev->cinMfma * es);
       if (rc != D3D_OK) return rc;
-      rc = launchPadRows(inputs[0], a.inRows, cin, dev->cinMfma, widened->ptr, stream);
+      rc = launchPadRows(inputs[0], a.inRows, cin * es, dev->cinMfma * es, widened->ptr, stream);
       if (rc != D3D_OK) return rc;
       a.in = widened->ptr;
       a.cin = dev->cinMfma;
@@ -721,7 +778,8 @@ struct MMPlugin final : d3d_plugin {
     a.out = outputs[0];
     a.weightsF32 = static_cast<const float*>(dev->f32.ptr);
     a.weightsMfma = dev->mfma.ptr;
-    a.bias = withBias ? static_cast<const float*>(dev->bias.ptr) : nullptr;
+    a.bias = (withBias || dtype == D3D_INT8) ? static_cast<const float*>(dev->bias.ptr) : nullptr;
+    a.requantM = dtype == D3D_INT8 ? static_cast<const float*>(dev->requantM.ptr) : nullptr;
     a.nbr = static_cast<const int32_t*>(table->ptr);
     a.relu = relu ? 1 : 0;
     a.zeros = zeros;

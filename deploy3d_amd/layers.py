@@ -52,7 +52,8 @@ class SparseConvLayer:
             spec["subm"], spec.get("transpose", False)))
         self.mm_plugin = Plugin("SPConvMM", mm_blob(
             spec["ksize"], spec["cin"], spec["cout"], self.max_num_act_out, spec["subm"], spec.get("inverse", False),
-            weight, bias, relu=spec.get("relu", False)))
+            weight, bias, relu=spec.get("relu", False), act_scale_in=float(spec.get("s_in", 1.0)),
+            act_scale_out=float(spec.get("s_out", 1.0))))
         self._idx_state = None
         self._mm_state = None
 
@@ -205,6 +206,7 @@ def measure_output_counts(layers, coords, grid, batch=1, device="cuda"):
 
 
 def make_input(coords, feats, grid, dtype=torch.float16, device="cuda", capacity=None, batch=1):
+    """Device tensors at capacity.  For torch.int8, ``feats`` must already be quantized int8 values."""
     n = len(coords)
     capacity = capacity or n
     c = torch.zeros((capacity, coords.shape[1]), dtype=torch.int32, device=device)

@@ -190,6 +190,37 @@ def config3(n=120000):
     return dict(config=3, grid=grid, coords=coords, feats=feats, dtype="float16", layers=layers, weights=weights)
 
 
+def activation_scale(a):
+    """Per-tensor symmetric int8 scale: the 99.99th percentile of |a| over 127, as float32."""
+    a = np.abs(np.asarray(a, dtype=np.float64)).reshape(-1)
+    s = np.percentile(a, 99.99) / 127.0 if a.size else 1.0
+    return np.float32(s if s > 0 else 1.0)
+
+
+def quantize_activations(a, scale):
+    return np.clip(np.rint(np.asarray(a, dtype=np.float64) / np.float64(scale)), -128, 127).astype(np.int8)
+
+
+def config4(n=120000, activations=None):
+    """Config 3 quantized to int8.  ``activations`` maps "input" and every layer name to that tensor's values
+    from a floating-point pass of config 3 at the same size (the calibration data); each layer gets the scales of
+    its input and output tensors as ``s_in`` / ``s_out``.  Weights stay fp32 in the blob: the engine derives the
+    per-output-channel weight scales itself."""
+    cfg = config3(n)
+    if activations is None:
+        raise ValueError("config4 needs the activations of a floating-point pass for calibration")
+    scales = {name: activation_scale(a) for name, a in activations.items()}
+    layers = []
+    prev = "input"
+    for spec in cfg["layers"]:
+        spec = dict(spec, s_in=scales[prev], s_out=scales[spec["name"]])
+        layers.append(spec)
+        prev = spec["name"]
+    cfg.update(config=4, dtype="int8", layers=layers, scales=scales,
+               feats_q=quantize_activations(cfg["feats"], scales["input"]))
+    return cfg
+
+
 def config5(n=250000):
     """Cylinder3D-style block on a cylindrical grid [rho, phi, z], fp16."""
     grid = (480, 360, 32)

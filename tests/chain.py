@@ -54,6 +54,23 @@ def oracle_chain(cfg, threads=1, acc="f64"):
         cur = dict(feats=round_to(y, dtype), exact=y, coords=rb["out_coors"], grid=rb["out_grid"],
                    pairs=rb["pairs"], key=spec["key"])
         outs[spec["name"]] = cur
+    outs["_rulebooks"] = rulebooks
+    return outs
+
+
+def oracle_chain_int8(cfg, rulebook_chain):
+    """Config-4 style chain in int8: ``cfg`` from synth.config4, ``rulebook_chain`` the result of oracle_chain on the
+    floating-point configuration (its rulebooks are reused: coordinates do not depend on the values).
+    Returns name -> int8 features [n, C] in the row order of rulebook_chain[name]["coords"]."""
+    outs = {"input": cfg["feats_q"]}
+    cur = outs["input"]
+    for spec, (w, b) in zip(cfg["layers"], cfg["weights"]):
+        rb = rulebook_chain["_rulebooks"][spec["key"]]
+        w_q, s_w = oracle.quantize_weights(w)
+        m, bq = oracle.requant_params(spec["s_in"], s_w, spec["s_out"], b)
+        acc = oracle.conv_i8(cur, w_q, rb["index"], rb["num_index"], rb["num_act_out"])
+        cur = oracle.requantize(acc, m, bq, bool(spec.get("relu")))
+        outs[spec["name"]] = cur
     return outs
 
 

@@ -80,6 +80,10 @@ def test_mm_blob_layout_and_round_trip():
     bad = list(ins)
     bad[0] = TensorDesc.of((500, 4), torch.int32)
     assert not p.supports_format(0, bad + [out], 5, 1)
+    q = list(ins)
+    q[0] = TensorDesc.of((500, 4), torch.int8)          # int8 features: this build's extension
+    assert p.supports_format(0, q + [out], 5, 1) and not p.supports_format(5, q + [out], 5, 1)
+    assert p.output_descs(q)[0].dtype == 2
     ext = mm_blob((3, 3, 3), 4, 8, 1000, True, False, w, b, relu=True)
     assert len(ext) == len(blob) + 20 and Plugin("SPConvMM", ext).serialize() == ext
 

@@ -97,6 +97,41 @@ def test_config3_backbone_reduced(engine):
     compare_chain(cfg, net, ref, tol_scale=1.5)  # 13 layers of fp16 rounding drift between two chains
 
 
+def _config4(n):
+    """Config 4 = config 3 quantized: calibration activations from a floating-point oracle pass at the same size."""
+    from deploy3d_amd import synth
+    cfg3 = synth.config3(n)
+    cfg3["dtype"] = "float32"
+    ref = chain.oracle_chain(cfg3, threads=8, acc="f32")
+    acts = {"input": cfg3["feats"]}
+    acts.update({s["name"]: ref[s["name"]]["exact"] for s in cfg3["layers"]})
+    return synth.config4(n, acts), ref
+
+
+def test_config4_int8_backbone_bit_exact(engine):
+    """Config 4 at 12 000 voxels: every layer's int8 output equals the oracle's (int32 accumulation + the written
+    requantize rule), row for row after sorting by coordinate."""
+    from deploy3d_amd import layers
+    n = 12000
+    cfg, ref = _config4(n)
+    want = chain.oracle_chain_int8(cfg, ref)
+    counts = layers.measure_output_counts(cfg["layers"], cfg["coords"], cfg["grid"])
+    caps = layers.plan_capacities(cfg["layers"], n, counts)
+    net = layers.SparseBackbone(cfg["layers"], cfg["weights"], caps, dtype=torch.int8)
+    x = layers.make_input(cfg["coords"], cfg["feats_q"], cfg["grid"], dtype=torch.int8)
+    net.forward(x)
+    torch.cuda.synchronize()
+    for spec in cfg["layers"]:
+        out = net.outputs[spec["name"]]
+        n_out = int(out.num_act.item())
+        assert n_out == len(ref[spec["name"]]["coords"])
+        gc, gf = chain.sort_rows(out.coors[:n_out].cpu().numpy(), out.feats[:n_out].cpu().numpy())
+        rc, rf = chain.sort_rows(ref[spec["name"]]["coords"], want[spec["name"]])
+        np.testing.assert_array_equal(gc, rc, err_msg=spec["name"])
+        np.testing.assert_array_equal(gf, rf, err_msg=spec["name"])
+        assert np.abs(rf.astype(np.int32)).max() >= 100, spec["name"]     # the calibrated range is in use
+
+
 def test_config3_backbone_full_size_properties(engine):
     """Config 3 at 120 000 voxels: size-independent checks (no oracle pass over 138 GFLOP)."""
     from deploy3d_amd import synth

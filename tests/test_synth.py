@@ -62,3 +62,13 @@ def test_bn_fold_matches_batchnorm_eval():
     want = bn(x @ torch.from_numpy(w_raw[0]))
     got = x @ torch.from_numpy(w[0]) + torch.from_numpy(b)
     assert torch.allclose(got, want, atol=1e-5)
+
+
+def test_int8_calibration_helpers():
+    a = np.linspace(-2.0, 2.0, 100001)
+    s = synth.activation_scale(a)
+    assert s.dtype == np.float32 and abs(float(s) - np.percentile(np.abs(a), 99.99) / 127) < 1e-7
+    s = np.float32(0.25)                                # exact in binary, so the ties below are exact ties
+    q = synth.quantize_activations(np.array([0.0, 0.125, 0.375, 0.625, -75.0, 75.0]), s)
+    assert q.tolist() == [0, 0, 2, 2, -128, 127]        # ties to even, clamp to the int8 range
+    assert synth.activation_scale(np.zeros(5)) == np.float32(1.0)
