@@ -21,9 +21,9 @@ METRIC = "sparse backbone latency ms + effective TFLOP/s, 120k voxels fp16, 1×M
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the roofline kernel at the default 120 000 voxels, from two `rocprofv3 --pmc` runs of this
-# script (FETCH_SIZE 33623, WRITE_SIZE 32778 per dispatch), each scaled by what the same counter read for the
+# script (FETCH_SIZE 33873, WRITE_SIZE 32768 per dispatch), each scaled by what the same counter read for the
 # 256 MiB copy of --pmc-copy-mib (FETCH_SIZE reads half the copied KiB: factor 2.0; WRITE_SIZE factor 1.0).
-MEASURED_TRAFFIC_BYTES = {("conv3", 120000): int((33623 * 2.0 + 32778 * 1.0) * 1024)}
+MEASURED_TRAFFIC_BYTES = {("conv3", 120000): int((33873 * 2.0 + 32768 * 1.0) * 1024)}
 
 
 def cpu_baseline(cfg, threads):
@@ -177,7 +177,7 @@ def main():
     dspec = specs[dom]
     achieved = layer_flops[dom] / (layer_ms[dom] * 1e-3) / 1e12
     roofline = {
-        "kernel": "convMfma<fp16,%d,%d> (layer %s)" % (dspec["cin"], dspec["cout"], dspec["name"]),
+        "kernel": "convStaged<fp16,%d,%d> (layer %s)" % (dspec["cin"], dspec["cout"], dspec["name"]),
         "bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES.get((dspec["name"][:5], args.voxels)),
