@@ -647,6 +647,14 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
     __syncthreads();
   }
 
+  // per-lane constants of the gathers: byte offset of this lane's (swizzled) chunk inside a row
+  uint32_t chunkOff[GL];
+#pragma unroll
+  for (int j = 0; j < GL; ++j)
+    chunkOff[j] = static_cast<uint32_t>(((lane % CH) ^ stageSwizzle<CH>(j * RPI + lane / CH)) * 16);
+  const uint32_t rowLimit = static_cast<uint32_t>(inRows);   // the launcher keeps inRows * row bytes below 4 GiB
+  const uintptr_t zeroBase = reinterpret_cast<uintptr_t>(zeros);
+
   const int perXcd = (tileBlocks + 7) / 8;
   const int xcd = blockIdx.x & 7;
   for (int local = blockIdx.x >> 3; local < perXcd; local += gridDim.x >> 3) {
@@ -668,19 +676,19 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
         __builtin_amdgcn_global_load_lds(wk + base + lane, wLds + buf * WCH + base, 16, 0, 0);
       }
     };
+    // Branch-free addresses: an absent neighbour (-1) or a row index past the input compares as a huge unsigned
+    // number and selects the zero row; rows past outRows repeat the last row's neighbours and are never stored.
     auto issueRows = [&](int t, int slot) __attribute__((always_inline)) {
       const int32_t* ix = idxLds + (t & (NI - 1)) * 64;
-      int32_t src[GL];
+      uint32_t src[GL];
 #pragma unroll
-      for (int j = 0; j < GL; ++j) src[j] = ix[j * RPI + lane / CH];
+      for (int j = 0; j < GL; ++j) src[j] = static_cast<uint32_t>(ix[j * RPI + lane / CH]);
+      const uintptr_t inBase = reinterpret_cast<uintptr_t>(in) + static_cast<uint32_t>((t % KS) * CS * ES);
 #pragma unroll
       for (int j = 0; j < GL; ++j) {
-        const int n = j * RPI + lane / CH;
-        const int c = (lane % CH) ^ stageSwizzle<CH>(n);
-        const bool ok = src[j] >= 0 && src[j] < inRows && row0 + n < outRows;
-        const T* p = (ok ? in + static_cast<size_t>(src[j]) * CIN + (t % KS) * CS : zeros) + c * EPC;
-        // (a half-precision pointer here makes the host pass drop the kernel's launch stub without a diagnostic)
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(p), stage + slot * SLOTS + j * 64, 16, 0, 0);
+        const uintptr_t row = inBase + static_cast<uint64_t>(src[j] * static_cast<uint32_t>(CIN * ES));
+        const uintptr_t a = (src[j] < rowLimit ? row : zeroBase) + chunkOff[j];
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(a), stage + slot * SLOTS + j * 64, 16, 0, 0);
       }
     };
 
@@ -726,18 +734,24 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot has been read before it is refilled
         issueRows(a + NS, slot);
       }
+      // every weight fragment of the step is requested before the first MFMA, so the MFMAs start as the
+      // fragments arrive instead of paying the LDS latency once per fragment pair
       const F* wTap = reinterpret_cast<const F*>(wLds + (RESIDENT ? a : wbuf) * WCH);
+      F wts[KK][NT];
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) wts[kk][n] = wTap[(kk * NT + n) * 64 + lane];
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
         for (int n = 0; n < NT; ++n) {
-          const F wfrag = wTap[(kk * NT + n) * 64 + lane];
 #pragma unroll
           for (int m = 0; m < MT; ++m) {
             if constexpr (WIDE) {
-              acc[m][n] = Mfma<T>::k32(wfrag, rows[m][kk], acc[m][n]);
+              acc[m][n] = Mfma<T>::k32(wts[kk][n], rows[m][kk], acc[m][n]);
             } else {
-              acc[m][n] = Mfma<T>::k16(wfrag, rows[m][kk], acc[m][n]);
+              acc[m][n] = Mfma<T>::k16(wts[kk][n], rows[m][kk], acc[m][n]);
             }
           }
         }
@@ -771,12 +785,17 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
         else if (allowed >= GL) waitVmcnt<cmin(GL, 63)>();
         else waitVmcnt<0>();
       }
-      if (!RESIDENT) __syncthreads();
+      // a bare barrier: __syncthreads() would also drain every load in flight, i.e. the whole prefetch
+      if (!RESIDENT) __builtin_amdgcn_s_barrier();
       slot = slot + 1 == NS ? 0 : slot + 1;
       wbuf = wbuf + 1 == NWB ? 0 : wbuf + 1;
     }
 
     // epilogue: bias, ReLU, rounding; rows leave through the stage area as contiguous lines
+    const float* biasRow = bias ? bias : reinterpret_cast<const float*>(zeros);  // the zero row doubles as "no bias"
+    float4v biasV[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) biasV[n] = *reinterpret_cast<const float4v*>(biasRow + n * 16 + kgrp * 4);
     if constexpr (LDS_EPILOGUE) {
       unsigned char* sb = reinterpret_cast<unsigned char*>(stage);
 #pragma unroll
@@ -788,7 +807,7 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
           float v[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            v[j] = acc[m][n][j] + (bias ? bias[col + j] : 0.f);
+            v[j] = acc[m][n][j] + biasV[n][j];
             if (relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
           }
           T packed[4] = {static_cast<T>(v[0]), static_cast<T>(v[1]), static_cast<T>(v[2]), static_cast<T>(v[3])};
@@ -819,7 +838,7 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             float t = static_cast<float>(acc[m][n][j]) * requantM[col + j];
-            t = t + (bias ? bias[col + j] : 0.f);
+            t = t + biasV[n][j];
             float q = __builtin_rintf(t);
             q = __builtin_fminf(127.f, __builtin_fmaxf(relu ? 0.f : -128.f, q));
             packed |= (static_cast<uint32_t>(static_cast<int>(q)) & 0xFFu) << (8 * j);
@@ -838,7 +857,7 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
           float v[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            v[j] = acc[m][n][j] + (bias ? bias[col + j] : 0.f);
+            v[j] = acc[m][n][j] + biasV[n][j];
             if (relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
           }
           T packed[4] = {static_cast<T>(v[0]), static_cast<T>(v[1]), static_cast<T>(v[2]), static_cast<T>(v[3])};
@@ -918,6 +937,7 @@ int32_t launchStagedCfg(const ConvArgs& a, hipStream_t stream) {
   const size_t lds = static_cast<size_t>(RESIDENT ? a.kVol * KS : 3) * WCH * 16 + static_cast<size_t>(WAVES) * 4 * 256 +
                      static_cast<size_t>(WAVES) * NS * WM * CH * 16;
   if (lds > kLdsLimit) return D3D_ERR_UNSUPPORTED;  // the caller falls back
+  if (static_cast<uint64_t>(a.inRows) * CIN * sizeof(T) >= (1ull << 32)) return D3D_ERR_UNSUPPORTED;  // 32-bit row offsets
   static size_t granted = 64 * 1024;
   const int32_t rc = grantLds(&convStaged<T, CIN, COUT, KS, MT, WAVES, NS, RESIDENT>, lds, &granted);
   if (rc != D3D_OK) return rc;
