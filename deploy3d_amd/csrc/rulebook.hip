@@ -545,8 +545,10 @@ __device__ __forceinline__ bool tapTargetCoord(const RbGeom& g, const int c[5], 
   return ok;
 }
 
-__device__ __forceinline__ uint32_t bmRank(const BmRecord& r, uint32_t bit) {
-  return r.prefix + static_cast<uint32_t>(__popcll(r.bits & ((1ull << bit) - 1ull)));
+// rank = occupied cells in earlier chunks of 1024 records + in earlier records of the chunk + below the bit
+__device__ __forceinline__ uint32_t bmRank(const BmRecord& r, uint32_t bit, const uint32_t* __restrict__ chunkBase,
+                                           uint32_t rec) {
+  return chunkBase[rec / kRbChunk] + r.prefix + static_cast<uint32_t>(__popcll(r.bits & ((1ull << bit) - 1ull)));
 }
 
 // reset for the block-map path: records = 0, index tensor = -1, counters = 0
@@ -649,36 +651,14 @@ bmMarkCandidates(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const 
   }
 }
 
-// Occupied cells per chunk of 1024 records.
+// One pass over the records: every record gets the count of occupied cells before it INSIDE its chunk of 1024
+// records, every chunk its total; the workgroup that finishes last (a ticket counter, no waiting) turns the chunk
+// totals into exclusive chunk bases and writes numActOut = min(total, maxNumActOut) for strided convolutions.
 __global__ void __launch_bounds__(kRbThreads)
-bmChunkTotals(const BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* __restrict__ chunkTotals) {
+bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, uint32_t nChunks, uint32_t* ticket,
+       int32_t* numActOut, int32_t maxNumActOut) {
   __shared__ uint32_t scratch[kRbThreads / 64];
-  const uint32_t first = blockIdx.x * kRbChunk + threadIdx.x * kRbItems;
-  uint32_t mine = 0;
-#pragma unroll
-  for (int j = 0; j < kRbItems; ++j)
-    if (first + j < nRecords) mine += static_cast<uint32_t>(__popcll(records[first + j].bits));
-  const uint32_t total = blockSum(mine, scratch);
-  if (threadIdx.x == 0) chunkTotals[blockIdx.x] = total;
-}
-
-// Writes every record's prefix, and numActOut = min(total, maxNumActOut) for strided convolutions.
-__global__ void __launch_bounds__(kRbThreads)
-bmPrefix(BmRecord* __restrict__ records, uint32_t nRecords, const uint32_t* __restrict__ chunkTotals,
-         uint32_t nChunks, int32_t* numActOut, int32_t maxNumActOut) {
-  __shared__ uint32_t scratch[kRbThreads / 64];
-  uint32_t before = 0, all = 0;
-  for (uint32_t q = threadIdx.x; q < nChunks; q += blockDim.x) {
-    const uint32_t v = chunkTotals[q];
-    if (q < blockIdx.x) before += v;
-    all += v;
-  }
-  const uint32_t base = blockSum(before, scratch);
-  if (blockIdx.x == 0 && numActOut) {
-    const uint32_t total = blockSum(all, scratch);
-    if (threadIdx.x == 0)
-      *numActOut = static_cast<int32_t>(total < static_cast<uint32_t>(maxNumActOut) ? total : maxNumActOut);
-  }
+  __shared__ uint32_t isLast;
   const uint32_t first = blockIdx.x * kRbChunk + threadIdx.x * kRbItems;
   uint32_t count[kRbItems];
   uint32_t mine = 0;
@@ -688,25 +668,46 @@ bmPrefix(BmRecord* __restrict__ records, uint32_t nRecords, const uint32_t* __re
     mine += count[j];
   }
   uint32_t total;
-  uint32_t rank = base + blockExclusiveScan(mine, scratch, &total);
+  uint32_t rank = blockExclusiveScan(mine, scratch, &total);
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
     if (first + j < nRecords) records[first + j].prefix = rank;
     rank += count[j];
   }
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(&chunkBase[blockIdx.x], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __threadfence();
+    isLast = atomicAdd(ticket, 1u) == nChunks - 1 ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!isLast) return;
+  __threadfence();
+  uint32_t running = 0;
+  for (uint32_t q0 = 0; q0 < nChunks; q0 += kRbThreads) {
+    const uint32_t q = q0 + threadIdx.x;
+    const uint32_t v = q < nChunks ? __hip_atomic_load(&chunkBase[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    uint32_t sum;
+    const uint32_t ex = blockExclusiveScan(v, scratch, &sum);
+    if (q < nChunks) chunkBase[q] = running + ex;
+    running += sum;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0 && numActOut)
+    *numActOut = static_cast<int32_t>(running < static_cast<uint32_t>(maxNumActOut) ? running : maxNumActOut);
 }
+
 
 // Strided convolutions: output coordinates in rank order (reference: coorsOutOrganizeKernel,
 // index.cu:104-121).  One wavefront per record, one lane per cell of the brick.
 __global__ void __launch_bounds__(kRbThreads)
-bmEmitCoords(RbGeom g, BlockMap m, const BmRecord* __restrict__ records, uint32_t nRecords,
-             int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
+bmEmitCoords(RbGeom g, BlockMap m, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+             uint32_t nRecords, int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
   const uint32_t rec = blockIdx.x * (kRbThreads / 64) + (threadIdx.x >> 6);
   if (rec >= nRecords) return;
   const BmRecord r = records[rec];
   uint32_t bit = threadIdx.x & 63;
   if (!((r.bits >> bit) & 1ull)) return;
-  const uint32_t id = bmRank(r, bit);
+  const uint32_t id = bmRank(r, bit, chunkBase, rec);
   if (id >= static_cast<uint32_t>(maxNumActOut)) return;
   const int pad = kMaxSpatial - g.nd;
   int32_t* row = outCoors + static_cast<size_t>(id) * (g.nd + 1);
@@ -726,8 +727,8 @@ bmEmitCoords(RbGeom g, BlockMap m, const BmRecord* __restrict__ records, uint32_
 // SubM: perm[rank of voxel i] = i (reference: the value side of setSubMHashKernel, index.cu:174-182).
 __global__ void __launch_bounds__(kRbThreads)
 bmPermutation(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn,
-              int64_t cap, const BmRecord* __restrict__ records, uint32_t* __restrict__ perm,
-              uint32_t* permShuffled) {
+              int64_t cap, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+              uint32_t* __restrict__ perm, uint32_t* permShuffled) {
   const int n = liveCount(numActIn, cap);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= n) return;
@@ -736,7 +737,7 @@ bmPermutation(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int
   if (!coordInGrid(g, c)) return;
   uint32_t rec, bit;
   bmLocate(m, c, &rec, &bit);
-  const uint32_t rank = bmRank(records[rec], bit);
+  const uint32_t rank = bmRank(records[rec], bit, chunkBase, rec);
   perm[rank] = static_cast<uint32_t>(i);
   // rows that already sit in rank order (the outputs of a strided rulebook of this engine do)
   // need no permutation lookups in the probe; any mismatch raises the flag
@@ -750,9 +751,9 @@ bmPermutation(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int
 template <bool SUBM>
 __global__ void __launch_bounds__(kRbThreads)
 bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
-        int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ perm,
-        const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
-        uint32_t* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
+        int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+        const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut,
+        uint32_t* __restrict__ staging, uint32_t* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
   const int tap = blockIdx.y;
@@ -775,7 +776,7 @@ bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* 
           bmLocate(m, o, &rec, &bit);
           const BmRecord r = records[rec];
           if ((r.bits >> bit) & 1ull) {
-            const uint32_t rank = bmRank(r, bit);
+            const uint32_t rank = bmRank(r, bit, chunkBase, rec);
             if (SUBM) {
               row[j] = shuffled ? perm[rank] : rank;
             } else if (rank < static_cast<uint32_t>(maxNumActOut)) {
@@ -921,9 +922,9 @@ bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_
 template <bool SUBM>
 __global__ void __launch_bounds__(kRbThreads)
 bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
-            int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ perm,
-            const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
-            uint32_t* cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
+            int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+            const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut,
+            uint32_t* __restrict__ staging, uint32_t* cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
             int64_t nFillB, uint32_t fillBlocks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char nearSmem[];
   uint4* group = reinterpret_cast<uint4*>(nearSmem);                                   // [8][kRbThreads] records
@@ -954,11 +955,17 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
   uint32_t rec[kNearGroup];
   const uint32_t present = live ? nearMembers(m, b, rec) : (nearMembers(m, b, rec), 0u);
   uint4 loaded[kNearGroup];
+  uint32_t base[kNearGroup];
 #pragma unroll
-  for (int e = 0; e < kNearGroup; ++e) loaded[e] = *reinterpret_cast<const uint4*>(records + (live ? rec[e] : 0u));
+  for (int e = 0; e < kNearGroup; ++e) {
+    loaded[e] = *reinterpret_cast<const uint4*>(records + (live ? rec[e] : 0u));
+    base[e] = chunkBase[(live ? rec[e] : 0u) / kRbChunk];
+  }
 #pragma unroll
-  for (int e = 0; e < kNearGroup; ++e)
+  for (int e = 0; e < kNearGroup; ++e) {
+    loaded[e].z += base[e];  // in-chunk prefix -> global prefix
     group[e * kRbThreads + threadIdx.x] = ((present >> e) & 1u) ? loaded[e] : make_uint4(0, 0, 0, 0);
+  }
   __syncthreads();  // ldsCnt zeroed
   nearForEachTap(g, m, c, b, [&](int tap, bool ok, int member, uint32_t bit) {
     uint32_t row = kNone;
@@ -1087,8 +1094,8 @@ RbWorkspace planWith(const RbGeom& g, int64_t cap, bool subM, bool blockMap) {
   off = alignUp(off + static_cast<size_t>(g.kVol) * w.pitch * 4);
   w.cnt = off;     // [kVol, nBlocks], directly followed (no gap) by
   off += static_cast<size_t>(g.kVol) * w.nBlocks * 4;
-  w.totals = off;  // [2, kVol] + 1: valid pairs per tap, owned outputs per tap, "rows not in rank order" flag
-  off = alignUp(off + (static_cast<size_t>(g.kVol) * 2 + 1) * 4);
+  w.totals = off;  // [2, kVol] + 2: valid pairs per tap, owned outputs per tap, "rows not in rank order" flag, scan ticket
+  off = alignUp(off + (static_cast<size_t>(g.kVol) * 2 + 2) * 4);
   w.total = off;
   return w;
 }
@@ -1190,14 +1197,15 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     const BlockMap m = makeBlockMap(g, &nRecords64);
     auto* records = reinterpret_cast<BmRecord*>(ws + w.table);
     auto* perm = reinterpret_cast<uint32_t*>(ws + w.ids);
-    auto* chunkTotals = reinterpret_cast<uint32_t*>(ws + w.ownCnt);
+    auto* chunkBase = reinterpret_cast<uint32_t*>(ws + w.ownCnt);
+    uint32_t* scanTicket = totals + 2 * g.kVol + 1;
     const dim3 perChunk(w.nChunks > 0 ? w.nChunks : 1);
     uint32_t* permShuffled = totals + 2 * g.kVol;
     const bool near = nearEligible(g, m);
     const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
     hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + (near ? 0 : nIndex / 4) + 1), block, 0,
                        stream, reinterpret_cast<uint4*>(records), static_cast<int64_t>(w.nRecords),
-                       near ? nullptr : index, nIndex, cnt, static_cast<int64_t>(g.kVol) * w.nBlocks + 2 * g.kVol + 1,
+                       near ? nullptr : index, nIndex, cnt, static_cast<int64_t>(g.kVol) * w.nBlocks + 2 * g.kVol + 2,
                        numIndex);
     if (subM) {
       hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
@@ -1206,15 +1214,14 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     } else {
       hipLaunchKernelGGL(bmMarkCandidates, perTap, block, 0, stream, g, m, coors, numActIn, cap, records);
     }
-    hipLaunchKernelGGL(bmChunkTotals, perChunk, block, 0, stream, records, w.nRecords, chunkTotals);
-    hipLaunchKernelGGL(bmPrefix, perChunk, block, 0, stream, records, w.nRecords, chunkTotals, w.nChunks,
+    hipLaunchKernelGGL(bmScan, perChunk, block, 0, stream, records, w.nRecords, chunkBase, w.nChunks, scanTicket,
                        subM ? nullptr : numActOut, maxNumActOut);
     if (!subM)
       hipLaunchKernelGGL(bmEmitCoords, dim3((w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64)), block, 0, stream,
-                         g, m, records, w.nRecords, outCoors, maxNumActOut);
+                         g, m, records, chunkBase, w.nRecords, outCoors, maxNumActOut);
     if (subM)
-      hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, perm,
-                         permShuffled);
+      hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, chunkBase,
+                         perm, permShuffled);
     if (near) {  // probe workgroups interleaved 3:1 with fill workgroups (index tensor, neighbour table)
       const uint32_t probeBlocks = perInput.x;
       const uint32_t quads = (probeBlocks + 2) / 3;
@@ -1224,18 +1231,18 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       nbrFilled = true;
       if (subM) {
         hipLaunchKernelGGL(bmProbeNear<true>, fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,
-                           records, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
+                           records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
                            fillB, nFillB, quads);
       } else {
         hipLaunchKernelGGL(bmProbeNear<false>, fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,
-                           records, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
+                           records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
                            fillB, nFillB, quads);
       }
     } else if (subM) {
-      hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, perm,
+      hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, chunkBase, perm,
                          permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
     } else {
-      hipLaunchKernelGGL(bmProbe<false>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, perm,
+      hipLaunchKernelGGL(bmProbe<false>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, chunkBase, perm,
                          permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
     }
   } else {
