@@ -453,7 +453,8 @@ __global__ void __launch_bounds__(kRbThreads)
 rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int kVol,
           const uint32_t* __restrict__ staging, const uint32_t* __restrict__ cnt, uint32_t nBlocks,
           const uint32_t* __restrict__ totals, int32_t* __restrict__ gather, int32_t* __restrict__ scatter,
-          int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* __restrict__ nbr, int64_t nbrRows) {
+          int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* __restrict__ nbr, int64_t nbrRows,
+          const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int tap = blockIdx.y;
   const uint32_t b = blockIdx.x;
@@ -474,7 +475,12 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
   const int64_t first = static_cast<int64_t>(b) * kRbChunk + threadIdx.x * kRbItems;
   uint4 s4 = make_uint4(kNone, kNone, kNone, kNone);
   if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<size_t>(tap) * pitch + first);
-  const uint32_t v[kRbItems] = {s4.x, s4.y, s4.z, s4.w};
+  uint32_t v[kRbItems] = {s4.x, s4.y, s4.z, s4.w};
+  if (perm && *permShuffled) {  // block-map SubM: the probe stored ranks; rows are perm[rank]
+#pragma unroll
+    for (int j = 0; j < kRbItems; ++j)
+      if (first + j < n && v[j] != kNone) v[j] = perm[v[j]];
+  }
   uint32_t mine = 0;
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) mine += (first + j < n && v[j] != kNone);
@@ -675,13 +681,15 @@ bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, u
     rank += count[j];
   }
   if (threadIdx.x == 0) {
-    __hip_atomic_store(&chunkBase[blockIdx.x], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __threadfence();
-    isLast = atomicAdd(ticket, 1u) == nChunks - 1 ? 1u : 0u;
+    // No fence (a device-scope release writes the L2 back, once per workgroup): the total is published with a
+    // returning device-scope atomic, which has been performed where every XCD sees it once its result is back,
+    // and only then is the ticket taken.
+    uint32_t old = __hip_atomic_exchange(&chunkBase[blockIdx.x], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(old)::"memory");
+    isLast = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nChunks - 1 ? 1u : 0u;
   }
   __syncthreads();
   if (!isLast) return;
-  __threadfence();
   uint32_t running = 0;
   for (uint32_t q0 = 0; q0 < nChunks; q0 += kRbThreads) {
     const uint32_t q = q0 + threadIdx.x;
@@ -699,10 +707,10 @@ bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, u
 
 // Strided convolutions: output coordinates in rank order (reference: coorsOutOrganizeKernel,
 // index.cu:104-121).  One wavefront per record, one lane per cell of the brick.
-__global__ void __launch_bounds__(kRbThreads)
-bmEmitCoords(RbGeom g, BlockMap m, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
-             uint32_t nRecords, int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
-  const uint32_t rec = blockIdx.x * (kRbThreads / 64) + (threadIdx.x >> 6);
+// outCoors[rank] = coordinate of every occupied cell of record `rec`; one wavefront per record, lane = cell
+__device__ __forceinline__ void emitRecordCoords(const RbGeom& g, const BlockMap& m, const BmRecord* __restrict__ records,
+                                                 const uint32_t* __restrict__ chunkBase, uint32_t nRecords, uint32_t rec,
+                                                 int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
   if (rec >= nRecords) return;
   const BmRecord r = records[rec];
   uint32_t bit = threadIdx.x & 63;
@@ -724,13 +732,20 @@ bmEmitCoords(RbGeom g, BlockMap m, const BmRecord* __restrict__ records, const u
   row[0] = static_cast<int32_t>(q);
 }
 
-// SubM: perm[rank of voxel i] = i (reference: the value side of setSubMHashKernel, index.cu:174-182).
 __global__ void __launch_bounds__(kRbThreads)
-bmPermutation(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn,
-              int64_t cap, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
-              uint32_t* __restrict__ perm, uint32_t* permShuffled) {
-  const int n = liveCount(numActIn, cap);
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+bmEmitCoords(RbGeom g, BlockMap m, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+             uint32_t nRecords, int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
+  emitRecordCoords(g, m, records, chunkBase, nRecords, blockIdx.x * (kRbThreads / 64) + (threadIdx.x >> 6), outCoors,
+                   maxNumActOut);
+}
+
+// SubM: perm[rank of voxel i] = i (reference: the value side of setSubMHashKernel, index.cu:174-182).
+// perm[rank] = input row i (SubM).  Rows that already sit in rank order (the outputs of a strided rulebook of
+// this engine do) need no permutation afterwards; any mismatch raises the flag.
+__device__ __forceinline__ void permuteRow(const RbGeom& g, const BlockMap& m, const int32_t* __restrict__ coors, int n,
+                                           int64_t i, const BmRecord* __restrict__ records,
+                                           const uint32_t* __restrict__ chunkBase, uint32_t* __restrict__ perm,
+                                           uint32_t* permShuffled) {
   if (i >= n) return;
   int c[5];
   loadCoord(coors, g.nd, i, c);
@@ -739,9 +754,15 @@ bmPermutation(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int
   bmLocate(m, c, &rec, &bit);
   const uint32_t rank = bmRank(records[rec], bit, chunkBase, rec);
   perm[rank] = static_cast<uint32_t>(i);
-  // rows that already sit in rank order (the outputs of a strided rulebook of this engine do)
-  // need no permutation lookups in the probe; any mismatch raises the flag
   if (rank != static_cast<uint32_t>(i)) *permShuffled = 1u;
+}
+
+__global__ void __launch_bounds__(kRbThreads)
+bmPermutation(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn,
+              int64_t cap, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+              uint32_t* __restrict__ perm, uint32_t* permShuffled) {
+  permuteRow(g, m, coors, liveCount(numActIn, cap), static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x, records,
+             chunkBase, perm, permShuffled);
 }
 
 // SubM probe / strided resolve on the block map: staging[tap, i] = output row of
@@ -757,7 +778,6 @@ bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* 
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
   const int tap = blockIdx.y;
-  const bool shuffled = SUBM && *permShuffled != 0;
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
   uint32_t found = 0;
   if (static_cast<int64_t>(blockIdx.x) * kRbChunk < n) {  // workgroup-uniform
@@ -778,7 +798,7 @@ bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* 
           if ((r.bits >> bit) & 1ull) {
             const uint32_t rank = bmRank(r, bit, chunkBase, rec);
             if (SUBM) {
-              row[j] = shuffled ? perm[rank] : rank;
+              row[j] = rank;  // the compaction turns ranks into rows through perm[] when rows are shuffled
             } else if (rank < static_cast<uint32_t>(maxNumActOut)) {
               row[j] = rank;
             }
@@ -923,14 +943,27 @@ template <bool SUBM>
 __global__ void __launch_bounds__(kRbThreads)
 bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
             int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
-            const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut,
-            uint32_t* __restrict__ staging, uint32_t* cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
-            int64_t nFillB, uint32_t fillBlocks) {
+            uint32_t* __restrict__ perm, uint32_t* permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
+            uint32_t* cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
+            int64_t nFillB, uint32_t fillBlocks, int32_t* __restrict__ outCoors, uint32_t nRecords) {
   extern __shared__ __attribute__((aligned(16))) unsigned char nearSmem[];
   uint4* group = reinterpret_cast<uint4*>(nearSmem);                                   // [8][kRbThreads] records
   uint32_t* ldsCnt = reinterpret_cast<uint32_t*>(group + kNearGroup * kRbThreads);    // [kVol]
   // Every fourth workgroup is a fill workgroup: the -1 fill of the index tensor and of the neighbour table is
   // bandwidth-bound, this pass latency-bound, and neither depends on the other, so they share one launch.
+  // Workgroups past the interleaved range carry the pass that only the compaction waits for: the rank -> row
+  // permutation (SubM) or the output coordinates (strided).
+  if (blockIdx.x >= fillBlocks * 4) {
+    const uint32_t e = blockIdx.x - fillBlocks * 4;
+    if (SUBM) {
+      permuteRow(g, m, coors, liveCount(numActIn, cap), static_cast<int64_t>(e) * kRbThreads + threadIdx.x, records,
+                 chunkBase, perm, permShuffled);
+    } else {
+      emitRecordCoords(g, m, records, chunkBase, nRecords, e * (kRbThreads / 64) + (threadIdx.x >> 6), outCoors,
+                       maxNumActOut);
+    }
+    return;
+  }
   const uint32_t quad = blockIdx.x >> 2, part = blockIdx.x & 3;
   if (part == 3) {
     if (quad < fillBlocks) {
@@ -946,7 +979,6 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
   const int64_t i0 = static_cast<int64_t>(probeBlock) * kRbThreads;
   if (i0 >= n) return;  // workgroup-uniform
   for (int t = threadIdx.x; t < g.kVol; t += blockDim.x) ldsCnt[t] = 0;
-  const bool shuffled = SUBM && *permShuffled != 0;  // rows are not already in rank order
   const int64_t i = i0 + threadIdx.x;
   const bool live = i < n;
   int c[5] = {0, 0, 0, 0, 0};
@@ -975,7 +1007,7 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
       if ((bits >> bit) & 1ull) {
         const uint32_t rank = v.z + static_cast<uint32_t>(__popcll(bits & ((1ull << bit) - 1ull)));
         if (SUBM) {
-          row = shuffled ? perm[rank] : rank;
+          row = rank;  // the compaction turns ranks into rows through perm[] when rows are shuffled
         } else if (rank < static_cast<uint32_t>(maxNumActOut)) {
           row = rank;
         }
@@ -1192,6 +1224,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   };
 
   bool nbrFilled = false;
+  const uint32_t* compactPerm = nullptr;      // block-map SubM: staging holds ranks, rows = perm[rank] when shuffled
+  const uint32_t* compactPermFlag = nullptr;
   if (w.blockMap) {
     uint64_t nRecords64;
     const BlockMap m = makeBlockMap(g, &nRecords64);
@@ -1201,6 +1235,10 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     uint32_t* scanTicket = totals + 2 * g.kVol + 1;
     const dim3 perChunk(w.nChunks > 0 ? w.nChunks : 1);
     uint32_t* permShuffled = totals + 2 * g.kVol;
+    if (subM) {
+      compactPerm = perm;
+      compactPermFlag = permShuffled;
+    }
     const bool near = nearEligible(g, m);
     const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
     hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + (near ? 0 : nIndex / 4) + 1), block, 0,
@@ -1216,27 +1254,30 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     }
     hipLaunchKernelGGL(bmScan, perChunk, block, 0, stream, records, w.nRecords, chunkBase, w.nChunks, scanTicket,
                        subM ? nullptr : numActOut, maxNumActOut);
-    if (!subM)
-      hipLaunchKernelGGL(bmEmitCoords, dim3((w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64)), block, 0, stream,
-                         g, m, records, chunkBase, w.nRecords, outCoors, maxNumActOut);
-    if (subM)
-      hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, chunkBase,
-                         perm, permShuffled);
+    if (!near) {  // the near probe launch carries these passes itself
+      if (!subM)
+        hipLaunchKernelGGL(bmEmitCoords, dim3((w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64)), block, 0, stream,
+                           g, m, records, chunkBase, w.nRecords, outCoors, maxNumActOut);
+      if (subM)
+        hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, chunkBase,
+                           perm, permShuffled);
+    }
     if (near) {  // probe workgroups interleaved 3:1 with fill workgroups (index tensor, neighbour table)
       const uint32_t probeBlocks = perInput.x;
       const uint32_t quads = (probeBlocks + 2) / 3;
-      const dim3 fused(quads * 4);
+      const uint32_t extra = subM ? probeBlocks : (w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64);
+      const dim3 fused(quads * 4 + extra);
       int32_t* fillB = (nbrOut && nbrRows > 0) ? nbrOut : nullptr;
       const int64_t nFillB = fillB ? static_cast<int64_t>(g.kVol) * nbrRows : 0;
       nbrFilled = true;
       if (subM) {
         hipLaunchKernelGGL(bmProbeNear<true>, fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,
                            records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
-                           fillB, nFillB, quads);
+                           fillB, nFillB, quads, outCoors, w.nRecords);
       } else {
         hipLaunchKernelGGL(bmProbeNear<false>, fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,
                            records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
-                           fillB, nFillB, quads);
+                           fillB, nFillB, quads, outCoors, w.nRecords);
       }
     } else if (subM) {
       hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, chunkBase, perm,
@@ -1272,7 +1313,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     hipLaunchKernelGGL(rbFillMinusOne, fillGrid(static_cast<int64_t>(g.kVol) * nbrRows / 4 + 1), block, 0, stream, nbrOut,
                        static_cast<int64_t>(g.kVol) * nbrRows);
   hipLaunchKernelGGL(rbCompact, perTap, block, 0, stream, numActIn, cap, w.pitch, g.kVol, staging, cnt, w.nBlocks,
-                     totals, index, index + rowLen, index + 2 * rowLen, numIndex, nbrRows > 0 ? nbrOut : nullptr, nbrRows);
+                     totals, index, index + rowLen, index + 2 * rowLen, numIndex, nbrRows > 0 ? nbrOut : nullptr, nbrRows,
+                     compactPerm, compactPermFlag);
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;
 }
