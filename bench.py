@@ -144,7 +144,7 @@ def main():
                 y = net.forward(x)
             stream.synchronize()
             ms = (time.perf_counter() - t0) * 1e3 / args.steps
-            mode = "eager" + ("" if args.no_overlap else ", rulebooks beside convolutions on a second stream")
+            mode = "eager" + ("" if args.no_overlap else ", rulebooks beside convolutions on two side streams")
         else:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
@@ -158,7 +158,7 @@ def main():
                 graph.replay()
             torch.cuda.synchronize()
             ms = (time.perf_counter() - t0) * 1e3 / args.steps
-            mode = "hip-graph replay" + ("" if args.no_overlap else ", rulebooks beside convolutions on a second stream")
+            mode = "hip-graph replay" + ("" if args.no_overlap else ", rulebooks beside convolutions on two side streams")
         same = bool(torch.equal(y.feats, ref_out))
         if args.pmc_copy_mib:
             src = torch.ones(args.pmc_copy_mib << 20, dtype=torch.uint8, device="cuda")

@@ -100,12 +100,13 @@ class SparseBackbone:
     """A chain (or small DAG, via ``src``) of SparseConvLayers sharing rulebooks by indice key.
 
     Rulebooks depend on coordinates only, convolutions on features and on their rulebook.  With ``overlap``
-    (the default) the rulebooks are enqueued on a second HIP stream and every convolution waits for the event
-    of its own rulebook, so the latency-bound index kernels of later stages run beside the MFMA kernels of
-    earlier ones.  The side stream forks from and joins into the caller's current stream, so a forward pass can
-    still be captured into one HIP graph (it then holds two parallel branches).  (A third stream for the SubM
-    rulebooks, which only depend on the strided ones, made hipStreamEndCapture crash in the runtime; the
-    single side stream is what is supported.)
+    (the default) the strided rulebooks, which feed each other, are enqueued on a second HIP stream, the SubM
+    rulebooks on a third, and every convolution waits for the event of its own rulebook: the latency-bound index
+    kernels of later stages run beside the MFMA kernels of earlier ones.  A SubM rulebook is ordered behind the
+    strided rulebook that wrote its coordinates through an event of the MAIN stream, recorded where the main
+    stream waited for that rulebook (an event edge straight from one side stream to the other made
+    hipStreamEndCapture crash in the runtime).  The side streams fork from and join into the caller's current
+    stream, so a forward pass can still be captured into one HIP graph (it then holds parallel branches).
     """
 
     def __init__(self, layers, weights, capacities, dtype=torch.float16, device="cuda", overlap=True):
@@ -118,14 +119,16 @@ class SparseBackbone:
     def forward(self, x):
         main = side = None
         if self.overlap:
-            if self._side is None:
-                self._side = torch.cuda.Stream()
+            if self._side is None:  # strided rulebooks feed each other; SubM rulebooks hang off them
+                self._side = {False: torch.cuda.Stream(), True: torch.cuda.Stream()}
             main, side = torch.cuda.current_stream(), self._side
             fork = torch.cuda.Event()
             fork.record(main)
-            side.wait_event(fork)
+            for st in side.values():
+                st.wait_event(fork)
         rulebooks = {}
         pending = {}
+        strided_coords = {}  # coordinate tensor written by a strided rulebook -> main-stream event after its wait
         outs = {"input": x}
         cur = x
         for spec, lyr in zip(self.specs, self.layers):
@@ -139,12 +142,22 @@ class SparseBackbone:
                 inp = outs[src]
             key = spec["key"]
             if side is not None and key not in rulebooks:
-                with torch.cuda.stream(side):
-                    rulebooks[key] = lyr.build_rulebook(inp)
+                subm = bool(spec["subm"])
+                st = side[subm]
+                if subm and id(inp.coors) in strided_coords:
+                    # order behind the strided rulebook that wrote these coordinates, carried by an event of the
+                    # main stream (recorded when the main stream waited for that rulebook)
+                    st.wait_event(strided_coords[id(inp.coors)])
+                with torch.cuda.stream(st):
+                    rb = rulebooks[key] = lyr.build_rulebook(inp)
                     pending[key] = torch.cuda.Event()
-                    pending[key].record(side)
+                    pending[key].record(st)
             if key in pending:
                 main.wait_event(pending.pop(key))
+                if not spec["subm"]:
+                    seen = torch.cuda.Event()
+                    seen.record(main)
+                    strided_coords[id(rulebooks[key].out_coors)] = seen
             cur = lyr.forward(inp, rulebooks)
             outs[spec["name"]] = cur
         self.rulebooks = rulebooks
