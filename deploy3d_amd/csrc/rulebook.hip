@@ -896,6 +896,60 @@ __device__ __forceinline__ void nearForEachTap(const RbGeom& g, const BlockMap& 
   }
 }
 
+// The same enumeration for the shapes that matter (3-D, dilation 1, not transposed, kernel sizes known at compile
+// time, strides powers of two): everything that depends on one dim only - validity, output cell, brick of the
+// group, bit part - is computed once per dim and tap position, the K1*K2*K3 taps are fully unrolled, and a tap
+// costs a handful of instructions instead of three calls of the general per-dim routine.
+template <int K1, int K2, int K3, class Fn>
+__device__ __forceinline__ void nearForEachTapFixed(const RbGeom& g, const BlockMap& m, const int c[5],
+                                                    const NearBase& b, Fn&& f) {
+  constexpr int KS[3] = {K1, K2, K3};
+  bool ok[3][3];
+  int member[3][3];
+  uint32_t part[3][3];
+#pragma unroll
+  for (int q = 0; q < 3; ++q) {
+    const int dim = q + 1;
+    const int st = g.s[dim];                  // 1, 2 or 4
+    const int ls = st >> 1 > 1 ? 2 : st >> 1; // log2
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      if (i < KS[q]) {
+        const int num = c[dim + 1] + g.p[dim] - i;
+        const int o = num >> ls;
+        ok[q][i] = num >= 0 && (num & (st - 1)) == 0 && o < g.shape[dim + 1];
+        member[q][i] = ((o >> m.shift[dim]) - b.brick[dim]) & 1;
+        part[q][i] = static_cast<uint32_t>(o) & ((1u << m.shift[dim]) - 1);
+      } else {
+        ok[q][i] = false;
+        member[q][i] = 0;
+        part[q][i] = 0;
+      }
+    }
+  }
+  const bool ok0 = b.ok && c[1] == 0;  // dim 0 is degenerate: extent 1, kernel 1
+#pragma unroll
+  for (int i1 = 0; i1 < K1; ++i1)
+#pragma unroll
+    for (int i2 = 0; i2 < K2; ++i2)
+#pragma unroll
+      for (int i3 = 0; i3 < K3; ++i3) {
+        const uint32_t bit = (((part[0][i1] << m.shift[2]) | part[1][i2]) << m.shift[3]) | part[2][i3];
+        f((i1 * K2 + i2) * K3 + i3, ok0 && ok[0][i1] && ok[1][i2] && ok[2][i3],
+          (member[0][i1] << 2) | (member[1][i2] << 1) | member[2][i3], bit);
+      }
+}
+
+// KSEL picks the enumeration: 0 = general, else a fixed kernel shape.
+template <int KSEL, class Fn>
+__device__ __forceinline__ void nearTaps(const RbGeom& g, const BlockMap& m, const int c[5], const NearBase& b, Fn&& f) {
+  if constexpr (KSEL == 1) nearForEachTapFixed<3, 3, 3>(g, m, c, b, f);
+  else if constexpr (KSEL == 2) nearForEachTapFixed<3, 1, 1>(g, m, c, b, f);
+  else if constexpr (KSEL == 3) nearForEachTapFixed<3, 1, 3>(g, m, c, b, f);
+  else if constexpr (KSEL == 4) nearForEachTapFixed<1, 3, 3>(g, m, c, b, f);
+  else nearForEachTap(g, m, c, b, f);
+}
+
 // Record indices of the 8 group members; members outside the grid are clamped to record 0 (so that every
 // load is unconditional and all eight issue back to back) and reported absent in the returned mask.
 __device__ __forceinline__ uint32_t nearMembers(const BlockMap& m, const NearBase& b, uint32_t rec[kNearGroup]) {
@@ -912,6 +966,7 @@ __device__ __forceinline__ uint32_t nearMembers(const BlockMap& m, const NearBas
 
 // Strided / transposed: one thread marks all candidate outputs of one input: per brick of its group one
 // atomicOr for each run of neighbouring lanes that target the same brick.
+template <int KSEL>
 __global__ void __launch_bounds__(kRbThreads)
 bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
            BmRecord* records) {
@@ -927,7 +982,7 @@ bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_
 #pragma unroll
   for (int e = 0; e < kNearGroup; ++e) masks[e][threadIdx.x] = 0ull;
   if (live)
-    nearForEachTap(g, m, c, b, [&](int, bool ok, int member, uint32_t bit) {
+    nearTaps<KSEL>(g, m, c, b, [&](int, bool ok, int member, uint32_t bit) {
       if (ok) masks[member][threadIdx.x] |= 1ull << bit;
     });
 #pragma unroll
@@ -939,7 +994,7 @@ bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_
 
 // SubM probe / strided resolve, one thread per input (see bmProbe for the per-pair form).
 // cnt is accumulated with atomics (four workgroups share one chunk of 1024 inputs) and must start at zero.
-template <bool SUBM>
+template <bool SUBM, int KSEL>
 __global__ void __launch_bounds__(kRbThreads)
 bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
             int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
@@ -949,12 +1004,12 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
   extern __shared__ __attribute__((aligned(16))) unsigned char nearSmem[];
   uint4* group = reinterpret_cast<uint4*>(nearSmem);                                   // [8][kRbThreads] records
   uint32_t* ldsCnt = reinterpret_cast<uint32_t*>(group + kNearGroup * kRbThreads);    // [kVol]
-  // Every fourth workgroup is a fill workgroup: the -1 fill of the index tensor and of the neighbour table is
+  // Every second workgroup is a fill workgroup: the -1 fill of the index tensor and of the neighbour table is
   // bandwidth-bound, this pass latency-bound, and neither depends on the other, so they share one launch.
   // Workgroups past the interleaved range carry the pass that only the compaction waits for: the rank -> row
   // permutation (SubM) or the output coordinates (strided).
-  if (blockIdx.x >= fillBlocks * 4) {
-    const uint32_t e = blockIdx.x - fillBlocks * 4;
+  if (blockIdx.x >= fillBlocks * 2) {
+    const uint32_t e = blockIdx.x - fillBlocks * 2;
     if (SUBM) {
       permuteRow(g, m, coors, liveCount(numActIn, cap), static_cast<int64_t>(e) * kRbThreads + threadIdx.x, records,
                  chunkBase, perm, permShuffled);
@@ -964,8 +1019,8 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
     }
     return;
   }
-  const uint32_t quad = blockIdx.x >> 2, part = blockIdx.x & 3;
-  if (part == 3) {
+  const uint32_t quad = blockIdx.x >> 1, part = blockIdx.x & 1;
+  if (part == 1) {
     if (quad < fillBlocks) {
       const int64_t tid = static_cast<int64_t>(quad) * kRbThreads + threadIdx.x;
       const int64_t stride = static_cast<int64_t>(fillBlocks) * kRbThreads;
@@ -974,7 +1029,7 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
     }
     return;
   }
-  const uint32_t probeBlock = quad * 3 + part;
+  const uint32_t probeBlock = quad;
   const int n = liveCount(numActIn, cap);
   const int64_t i0 = static_cast<int64_t>(probeBlock) * kRbThreads;
   if (i0 >= n) return;  // workgroup-uniform
@@ -999,7 +1054,9 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
     group[e * kRbThreads + threadIdx.x] = ((present >> e) & 1u) ? loaded[e] : make_uint4(0, 0, 0, 0);
   }
   __syncthreads();  // ldsCnt zeroed
-  nearForEachTap(g, m, c, b, [&](int tap, bool ok, int member, uint32_t bit) {
+  uint32_t mine = 0;  // lane t of a wavefront counts the wavefront's pairs of tap t (t + 64 for more than 64 taps)
+  const int lane = threadIdx.x & 63;
+  nearTaps<KSEL>(g, m, c, b, [&](int tap, bool ok, int member, uint32_t bit) {
     uint32_t row = kNone;
     if (live && ok) {
       const uint4 v = group[member * kRbThreads + threadIdx.x];
@@ -1014,9 +1071,14 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
       }
     }
     if (live) staging[static_cast<size_t>(tap) * pitch + i] = row;
-    const unsigned long long hit = __ballot(row != kNone);
-    if ((threadIdx.x & 63) == 0 && hit) atomicAdd(&ldsCnt[tap], static_cast<uint32_t>(__popcll(hit)));
+    const uint32_t hits = static_cast<uint32_t>(__popcll(__ballot(row != kNone)));
+    if (KSEL != 0) {
+      if (lane == tap) mine += hits;           // tap is a compile-time constant below 64 here
+    } else if ((threadIdx.x & 63) == 0 && hits) {
+      atomicAdd(&ldsCnt[tap], hits);
+    }
   });
+  if (KSEL != 0 && mine) atomicAdd(&ldsCnt[lane], mine);
   __syncthreads();
   const uint32_t chunk = probeBlock / kRbItems;
   for (int t = threadIdx.x; t < g.kVol; t += blockDim.x) {
@@ -1143,6 +1205,22 @@ bool nearEligible(const RbGeom& g, const BlockMap& m) {
   return !(e && e[0] == '0');
 }
 
+// 1: 3x3x3, 2: 3x1x1, 3: 3x1x3, 4: 1x3x3 (3-D, dilation 1, strides 1/2/4, not transposed), else 0 = general code.
+// D3D_RULEBOOK_FIXED=0 forces the general enumeration (tests).
+int fixedKernelShape(const RbGeom& g) {
+  const char* e = std::getenv("D3D_RULEBOOK_FIXED");
+  if (e && e[0] == '0') return 0;
+  if (g.nd != 3 || g.transpose || g.k[0] != 1) return 0;
+  for (int dim = 1; dim < kMaxSpatial; ++dim)
+    if (g.d[dim] != 1 || (g.s[dim] != 1 && g.s[dim] != 2 && g.s[dim] != 4)) return 0;
+  const int k1 = g.k[1], k2 = g.k[2], k3 = g.k[3];
+  if (k1 == 3 && k2 == 3 && k3 == 3) return 1;
+  if (k1 == 3 && k2 == 1 && k3 == 1) return 2;
+  if (k1 == 3 && k2 == 1 && k3 == 3) return 3;
+  if (k1 == 1 && k2 == 3 && k3 == 3) return 4;
+  return 0;
+}
+
 bool blockMapFits(const RbGeom& g) {
   uint64_t records;
   makeBlockMap(g, &records);
@@ -1240,6 +1318,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       compactPermFlag = permShuffled;
     }
     const bool near = nearEligible(g, m);
+    const int ksel = near ? fixedKernelShape(g) : 0;
     const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
     hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + (near ? 0 : nIndex / 4) + 1), block, 0,
                        stream, reinterpret_cast<uint4*>(records), static_cast<int64_t>(w.nRecords),
@@ -1248,7 +1327,13 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     if (subM) {
       hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
     } else if (near) {
-      hipLaunchKernelGGL(bmMarkNear, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
+      switch (ksel) {
+        case 1: hipLaunchKernelGGL(bmMarkNear<1>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records); break;
+        case 2: hipLaunchKernelGGL(bmMarkNear<2>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records); break;
+        case 3: hipLaunchKernelGGL(bmMarkNear<3>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records); break;
+        case 4: hipLaunchKernelGGL(bmMarkNear<4>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records); break;
+        default: hipLaunchKernelGGL(bmMarkNear<0>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
+      }
     } else {
       hipLaunchKernelGGL(bmMarkCandidates, perTap, block, 0, stream, g, m, coors, numActIn, cap, records);
     }
@@ -1262,23 +1347,36 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
         hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, chunkBase,
                            perm, permShuffled);
     }
-    if (near) {  // probe workgroups interleaved 3:1 with fill workgroups (index tensor, neighbour table)
+    if (near) {  // probe workgroups interleaved 1:1 with fill workgroups (index tensor, neighbour table)
       const uint32_t probeBlocks = perInput.x;
-      const uint32_t quads = (probeBlocks + 2) / 3;
+      const uint32_t quads = probeBlocks;
       const uint32_t extra = subM ? probeBlocks : (w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64);
-      const dim3 fused(quads * 4 + extra);
+      const dim3 fused(quads * 2 + extra);
       int32_t* fillB = (nbrOut && nbrRows > 0) ? nbrOut : nullptr;
       const int64_t nFillB = fillB ? static_cast<int64_t>(g.kVol) * nbrRows : 0;
       nbrFilled = true;
+#define D3D_LAUNCH_PROBE_NEAR(SUBM, KSEL)                                                                          \
+  hipLaunchKernelGGL((bmProbeNear<SUBM, KSEL>), fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,   \
+                     records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index,    \
+                     nIndex, fillB, nFillB, quads, outCoors, w.nRecords)
       if (subM) {
-        hipLaunchKernelGGL(bmProbeNear<true>, fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,
-                           records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
-                           fillB, nFillB, quads, outCoors, w.nRecords);
+        switch (ksel) {
+          case 1: D3D_LAUNCH_PROBE_NEAR(true, 1); break;
+          case 2: D3D_LAUNCH_PROBE_NEAR(true, 2); break;
+          case 3: D3D_LAUNCH_PROBE_NEAR(true, 3); break;
+          case 4: D3D_LAUNCH_PROBE_NEAR(true, 4); break;
+          default: D3D_LAUNCH_PROBE_NEAR(true, 0);
+        }
       } else {
-        hipLaunchKernelGGL(bmProbeNear<false>, fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,
-                           records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index, nIndex,
-                           fillB, nFillB, quads, outCoors, w.nRecords);
+        switch (ksel) {
+          case 1: D3D_LAUNCH_PROBE_NEAR(false, 1); break;
+          case 2: D3D_LAUNCH_PROBE_NEAR(false, 2); break;
+          case 3: D3D_LAUNCH_PROBE_NEAR(false, 3); break;
+          case 4: D3D_LAUNCH_PROBE_NEAR(false, 4); break;
+          default: D3D_LAUNCH_PROBE_NEAR(false, 0);
+        }
       }
+#undef D3D_LAUNCH_PROBE_NEAR
     } else if (subM) {
       hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, chunkBase, perm,
                          permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);

@@ -13,13 +13,15 @@ from oracle import oracle
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["blockmap", "blockmap-per-pair", "hash"])
+@pytest.fixture(autouse=True, params=["blockmap", "blockmap-general", "blockmap-per-pair", "hash"])
 def structure(request, monkeypatch):
     """Every case runs on every rulebook variant: the dense block map with one thread per input (default whenever
-    the map fits and a kernel's reach is at most one brick), the block map with one thread per (tap, input) pair
-    (long-reach kernels, 4-D) and the open-addressing hash (grids too large for the map)."""
+    the map fits and a kernel's reach is at most one brick; 3x3x3, 3x1x1, 3x1x3 and 1x3x3 kernels take a tap
+    enumeration specialised at compile time, "general" switches that off), the block map with one thread per
+    (tap, input) pair (long-reach kernels, 4-D) and the open-addressing hash (grids too large for the map)."""
     monkeypatch.setenv("D3D_RULEBOOK", request.param.split("-")[0])
     monkeypatch.setenv("D3D_RULEBOOK_NEAR", "0" if request.param.endswith("per-pair") else "1")
+    monkeypatch.setenv("D3D_RULEBOOK_FIXED", "0" if request.param.endswith("general") else "1")
     return request.param
 
 SUBM_CASES = [
