@@ -677,7 +677,7 @@ bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, u
   uint32_t rank = blockExclusiveScan(mine, scratch, &total);
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
-    if (first + j < nRecords) records[first + j].prefix = rank;
+    if (count[j]) records[first + j].prefix = rank;  // an empty record is never ranked: on sparse grids most are
     rank += count[j];
   }
   if (threadIdx.x == 0) {
