@@ -690,13 +690,26 @@ bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, u
   }
   __syncthreads();
   if (!isLast) return;
+  // one exclusive scan over all chunk totals: thread t takes a contiguous run of them (all loads in flight at
+  // once), scans it in registers, and a single workgroup scan of the run sums supplies the offsets
+  constexpr uint32_t kRun = 8;
   uint32_t running = 0;
-  for (uint32_t q0 = 0; q0 < nChunks; q0 += kRbThreads) {
-    const uint32_t q = q0 + threadIdx.x;
-    const uint32_t v = q < nChunks ? __hip_atomic_load(&chunkBase[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+  for (uint32_t base = 0; base < nChunks; base += kRun * kRbThreads) {
+    const uint32_t q0 = base + threadIdx.x * kRun;
+    uint32_t v[kRun];
+#pragma unroll
+    for (uint32_t j = 0; j < kRun; ++j)
+      v[j] = q0 + j < nChunks ? __hip_atomic_load(&chunkBase[q0 + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    uint32_t mineSum = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < kRun; ++j) mineSum += v[j];
     uint32_t sum;
-    const uint32_t ex = blockExclusiveScan(v, scratch, &sum);
-    if (q < nChunks) chunkBase[q] = running + ex;
+    uint32_t at = running + blockExclusiveScan(mineSum, scratch, &sum);
+#pragma unroll
+    for (uint32_t j = 0; j < kRun; ++j) {
+      if (q0 + j < nChunks) chunkBase[q0 + j] = at;
+      at += v[j];
+    }
     running += sum;
     __syncthreads();
   }
