@@ -110,4 +110,19 @@ bool convUsesMfma(int32_t dtype, int cin, int cout);
 int paddedMfmaChannels(int32_t dtype, int cin, int cout);
 int32_t launchPadRows(const void* in, int64_t rows, int inBytes, int outBytes, void* out, hipStream_t stream);
 
+// Sparse rows -> dense [B, C, Z, Y, X] map (densify.hip).  The workspace holds one int32 per cell.
+struct DensifyArgs {
+  const void* feats;      // [cap, C] elements of elemBytes bytes
+  const int32_t* coors;   // [cap, 4] (b, z, y, x)
+  const int32_t* numAct;  // device int32[1], live rows
+  int32_t cap;
+  int C, elemBytes;
+  int B, Z, Y, X;
+  void* out;
+  void* workspace;
+  size_t workspaceBytes;
+};
+size_t densifyWorkspaceBytes(int64_t B, int64_t Z, int64_t Y, int64_t X);
+int32_t launchDensify(const DensifyArgs& a, hipStream_t stream);
+
 }  // namespace d3d

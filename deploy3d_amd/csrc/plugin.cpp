@@ -789,12 +789,122 @@ struct MMPlugin final : d3d_plugin {
   }
 };
 
+// --- BEVDensify --------------------------------------------------------------
+// Attribute layout: BEVDensifyPluginParam, one int32 outChannels
+// (trt/spconv/bev_densify_trt.cu:43-47; written by
+// deploy3d/symfun/ops/spconv/bev_densify.py:38).
+struct DensifyPlugin final : d3d_plugin {
+  int32_t outChannels = 0;
+
+  static int32_t parse(const void* data, size_t len, DensifyPlugin** out) {
+    if (!data || len < 4) {
+      setError("BEVDensify: attribute blob of %zu bytes, 4 expected", len);
+      return D3D_ERR_BAD_BLOB;
+    }
+    auto p = std::unique_ptr<DensifyPlugin>(new DensifyPlugin());
+    p->type = "BEVDensify";
+    std::memcpy(&p->outChannels, data, 4);
+    if (p->outChannels < 0) {
+      setError("BEVDensify: outChannels %d", p->outChannels);
+      return D3D_ERR_BAD_BLOB;
+    }
+    p->blob.assign(static_cast<const uint8_t*>(data), static_cast<const uint8_t*>(data) + len);
+    *out = p.release();
+    return D3D_OK;
+  }
+
+  d3d_plugin* clone() const override { return new DensifyPlugin(*this); }
+  int32_t numOutputs() const override { return 1; }
+  // [B, outChannels, Y, X] from inSpatialShape [B, 0, Z, Y, X] (bev_densify_trt.cu:86-97)
+  int32_t outputDims(int32_t idx, const d3d_tensor_desc* in, int32_t nbIn, d3d_tensor_desc* out) const override {
+    if (idx != 0 || !out || !in || nbIn < 4 || in[3].nb_dims != 5) return D3D_ERR_BAD_ARG;
+    std::memset(out, 0, sizeof(*out));
+    out->format = D3D_LINEAR;
+    out->nb_dims = 4;
+    out->dims[0] = in[3].dims[0];
+    out->dims[1] = outChannels;
+    out->dims[2] = in[3].dims[3];
+    out->dims[3] = in[3].dims[4];
+    return D3D_OK;
+  }
+  int32_t outputDtype(int32_t, const int32_t* inTypes, int32_t nbIn) const override {
+    return (inTypes && nbIn > 0) ? inTypes[0] : D3D_ERR_BAD_ARG;  // bev_densify_trt.cu:98-100
+  }
+  // The reference takes float and half features (bev_densify_trt.cu:101-115); bf16 and int8 rows move the same way.
+  static bool featureType(int32_t t) { return t == D3D_HALF || t == D3D_FLOAT || t == D3D_BF16 || t == D3D_INT8; }
+  int32_t supportsFormat(int32_t pos, const d3d_tensor_desc* io, int32_t nbIn, int32_t nbOut) const override {
+    if (!io || pos < 0 || pos >= nbIn + nbOut || io[pos].format != D3D_LINEAR) return 0;
+    if (pos == 0) return featureType(io[0].dtype);
+    if (pos <= 3) return io[pos].dtype == D3D_INT32;
+    return io[pos].dtype == io[0].dtype;
+  }
+  int32_t configure(const d3d_tensor_desc*, int32_t, const d3d_tensor_desc*, int32_t) override { return D3D_OK; }
+  // One int32 per cell of the grid: the cell -> row table.  (The reference needs none, bev_densify_trt.cu:130-135;
+  // it pays with a clearing pass and channel-strided stores instead.)
+  size_t workspaceSize(const d3d_tensor_desc* in, int32_t nbIn) const override {
+    if (!in || nbIn < 4 || in[3].nb_dims != 5) return 0;
+    return densifyWorkspaceBytes(in[3].dims[0], in[3].dims[2], in[3].dims[3], in[3].dims[4]);
+  }
+  int32_t enqueue(const d3d_tensor_desc* inDesc, const d3d_tensor_desc* outDesc, const void* const* inputs,
+                  void* const* outputs, void* workspace, size_t workspaceBytes, hipStream_t stream) override {
+    if (!inDesc || !outDesc || !inputs || !outputs) return D3D_ERR_BAD_ARG;
+    if (inDesc[0].nb_dims != 2 || inDesc[1].nb_dims != 2 || inDesc[1].dims[1] != 4 || inDesc[3].nb_dims != 5 ||
+        inDesc[1].dims[0] < inDesc[0].dims[0]) {
+      setError("BEVDensify: expects inFeats [cap, C], inCoors [cap, 4], numActIn [1], inSpatialShape [B, 0, Z, Y, X]");
+      return D3D_ERR_BAD_ARG;
+    }
+    const int32_t dtype = inDesc[0].dtype;
+    if (!featureType(dtype)) {
+      setError("BEVDensify: feature dtype %d not implemented", dtype);
+      return D3D_ERR_UNSUPPORTED;
+    }
+    const int64_t cap = inDesc[0].dims[0], C = inDesc[0].dims[1];
+    const int64_t B = inDesc[3].dims[0], Z = inDesc[3].dims[2], Y = inDesc[3].dims[3], X = inDesc[3].dims[4];
+    if (B < 0 || Z < 0 || Y < 0 || X < 0 || cap > 0x7fffffff || C > 0x7fffffff || B > 0x7fffffff || Z > 0x7fffffff ||
+        Y > 0x7fffffff || X > 0x7fffffff) {
+      setError("BEVDensify: tensor extents out of range");
+      return D3D_ERR_BAD_ARG;
+    }
+    // The map is addressed as [B, C, Z, Y, X] and handed on as [B, outChannels, Y, X] (bev_densify_trt.cu:160-163).
+    if (C * Z != outChannels) {
+      setError("BEVDensify: outChannels %d but the input has %lld channels on %lld levels", outChannels,
+               static_cast<long long>(C), static_cast<long long>(Z));
+      return D3D_ERR_BAD_ARG;
+    }
+    if (outDesc[0].nb_dims != 4 || outDesc[0].dims[0] != B || outDesc[0].dims[1] != outChannels ||
+        outDesc[0].dims[2] != Y || outDesc[0].dims[3] != X || outDesc[0].dtype != dtype) {
+      setError("BEVDensify: output must be [B, outChannels, Y, X] of the feature type");
+      return D3D_ERR_BAD_ARG;
+    }
+    if (B * C * Z * Y * X == 0) return D3D_OK;
+    if (!outputs[0] || !inputs[2] || (cap > 0 && (!inputs[0] || !inputs[1]))) {
+      setError("BEVDensify: null tensor pointer");
+      return D3D_ERR_BAD_ARG;
+    }
+    DensifyArgs a{};
+    a.feats = inputs[0];
+    a.coors = static_cast<const int32_t*>(inputs[1]);
+    a.numAct = static_cast<const int32_t*>(inputs[2]);
+    a.cap = static_cast<int32_t>(cap);
+    a.C = static_cast<int>(C);
+    a.elemBytes = dtypeBytes(dtype);
+    a.B = static_cast<int>(B);
+    a.Z = static_cast<int>(Z);
+    a.Y = static_cast<int>(Y);
+    a.X = static_cast<int>(X);
+    a.out = outputs[0];
+    a.workspace = workspace;
+    a.workspaceBytes = workspaceBytes;
+    return launchDensify(a, stream);
+  }
+};
+
 struct OpEntry {
   const char* name;
-  int nd;  // 0 = SPConvMM
+  int nd;  // 0 = SPConvMM, -1 = BEVDensify
 };
 constexpr OpEntry kOps[] = {{"SPConvIdx1d", 1}, {"SPConvIdx2d", 2}, {"SPConvIdx3d", 3}, {"SPConvIdx4d", 4},
-                            {"SPConvMM", 0}};
+                            {"SPConvMM", 0},    {"BEVDensify", -1}};
 constexpr const char* kVersion = "2.0";
 
 }  // namespace
@@ -832,6 +942,12 @@ int32_t d3d_create(const char* name, const char* version, const void* blob, size
   }
   for (const OpEntry& op : kOps) {
     if (std::strcmp(name, op.name) != 0) continue;
+    if (op.nd < 0) {
+      DensifyPlugin* p = nullptr;
+      int32_t rc = DensifyPlugin::parse(blob, len, &p);
+      *out = p;
+      return rc;
+    }
     if (op.nd == 0) {
       MMPlugin* p = nullptr;
       int32_t rc = MMPlugin::parse(blob, len, &p);

@@ -29,6 +29,15 @@ class SparseTensor:
         return self.coors.shape[0]
 
 
+def densify(x):
+    """[B, C*Z, Y, X] map of a SparseTensor (the step between a sparse backbone and a 2-D head,
+    reference: deploy3d/symfun/ops/spconv/bev_densify.py:18-45)."""
+    from .bev_densify import bev_densify
+    z, y, xdim = x.grid
+    shape = torch.empty((x.batch, 0, z, y, xdim), dtype=torch.int32, device=x.feats.device)
+    return bev_densify(x.feats, x.coors, x.num_act, shape, x.feats.shape[1] * z)
+
+
 class Rulebook:
     """Outputs of one SPConvIdx enqueue, cached under an indice key."""
 

@@ -1,7 +1,8 @@
 /* C ABI of the MI355X sparse-convolution engine.
  *
- * The library exposes the two operators of deploy3d's sparse-convolution path
- * as opaque plugin objects with the life cycle TensorRT drives on the
+ * The library exposes the operators of deploy3d's sparse-convolution path (the
+ * rulebook builder, the gather-GEMM-scatter, and the sparse-to-dense step that
+ * ends the sparse part of a network) as opaque plugin objects with the life cycle TensorRT drives on the
  * reference's IPluginV2DynamicExt classes: deserialize -> clone -> configure
  * -> workspace size -> enqueue (stream-ordered) -> destroy.  Every function is
  * noexcept, takes plain pointers and sizes, and returns an int32 status.
@@ -9,6 +10,7 @@
  * Operator names, version and the packed attribute blobs are the reference's:
  *   "SPConvIdx1d" .. "SPConvIdx4d", version "2.0"   (trt/spconv/index_trt.cu:20-50, :287-290)
  *   "SPConvMM",                     version "2.0"   (trt/spconv/mm_trt.cu:22-37, :239)
+ *   "BEVDensify",                   version "2.0"   (trt/spconv/bev_densify_trt.cu:37-47, :209)
  */
 #ifndef D3D_SPCONV_H_
 #define D3D_SPCONV_H_
@@ -61,7 +63,8 @@ typedef struct d3d_plugin d3d_plugin;
  *                  optionally followed by a 20-byte extension record
  *                  {u32 magic 'D3DX'; u32 version 1; u32 flags (bit0 fused ReLU);
  *                   f32 actScaleIn; f32 actScaleOut} that the reference's parser
- *                  skips as trailing floats. */
+ *                  skips as trailing floats.
+ *   BEVDensify:    int32 outChannels  (trt/spconv/bev_densify_trt.cu:43-47, :199-204) */
 int32_t d3d_create(const char* name, const char* version, const void* blob, size_t len, d3d_plugin** out);
 
 /* IPluginV2DynamicExt::clone (index_trt.cu:75-79, mm_trt.cu:75-79): clones share device weights. */
@@ -113,7 +116,14 @@ size_t d3d_workspace_size(const d3d_plugin* p, const d3d_tensor_desc* in, int32_
  *                         4 outSpatialShape (dims only)
  * SPConvMM       inputs : 0 inFeats [capIn, Cin], 1 numActIn [1], 2 numActOut [1],
  *                         3 index int32 [3, L], 4 numIndex int32 [1]
- *                outputs: 0 outFeats [maxNumActOut, Cout], dtype of input 0 */
+ *                outputs: 0 outFeats [maxNumActOut, Cout], dtype of input 0
+ * BEVDensify     (bev_densify_trt.cu:136-176; float, half, and also bf16 / int8 rows)
+ *                inputs : 0 inFeats [cap, C], 1 inCoors int32 [cap, 4] (b, z, y, x), 2 numActIn int32 [1],
+ *                         3 inSpatialShape (dims [B, 0, Z, Y, X] only; pointer unused)
+ *                outputs: 0 outFeatMaps [B, outChannels = C*Z, Y, X], dtype of input 0: zero except
+ *                         out[b, c*Z + z, y, x] = inFeats[i, c] for live row i at (b, z, y, x)
+ *                workspace: one int32 per grid cell (the reference needs none); rows outside the grid
+ *                         are skipped, and of rows naming one cell the highest stays */
 int32_t d3d_enqueue(d3d_plugin* p, const d3d_tensor_desc* in_desc, const d3d_tensor_desc* out_desc,
                     const void* const* inputs, void* const* outputs, void* workspace, size_t workspace_bytes,
                     void* stream);

@@ -146,6 +146,20 @@ def requant_params(s_in, s_w, s_out, bias):
     return m, bq
 
 
+def bev_densify(in_feats, in_coors, num_act_in, spatial_shape):
+    """Dense map [B, C*Z, Y, X] of the first num_act_in rows; spatial_shape = (B, Z, Y, X).
+    in_feats may be any 1/2/4-byte numpy dtype (fp16 as np.float16, bf16 as its uint16 bits)."""
+    in_feats = np.ascontiguousarray(in_feats)
+    in_coors = np.ascontiguousarray(in_coors, dtype=np.int32)
+    b, z, y, x = (int(v) for v in spatial_shape)
+    c = in_feats.shape[1]
+    out = np.empty((b, c * z, y, x), dtype=in_feats.dtype)
+    lib().d3d_oracle_bev_densify(_p(in_feats), _p(in_coors), ctypes.c_int32(int(num_act_in)), ctypes.c_int(c),
+                                 ctypes.c_int(in_feats.dtype.itemsize), ctypes.c_int(b), ctypes.c_int(z),
+                                 ctypes.c_int(y), ctypes.c_int(x), _p(out))
+    return out
+
+
 def canonical(index, num_index, out_coors, num_act_out):
     """Canonical form of a rulebook: output coordinates sorted lexicographically,
     scatter ids relabelled by that rank, triples (tap, gather, scatter) sorted.

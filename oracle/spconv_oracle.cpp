@@ -21,6 +21,8 @@
 //                  NOT in the reference (trt/spconv/mm_trt.cu:184 accepts fp16
 //                  only): parity unpinned by the reference, pinned only by the
 //                  written rule restated above requantize() below.
+//   bev_densify    the dense-indexing ground truth of the reference's own test
+//                  (tests/spconv/test_bev_densify.py:19-23) on its six cases
 //
 // Build: make -C oracle   (g++ -O2 -fopenmp -ffp-contract=off)
 #include <algorithm>
@@ -352,6 +354,23 @@ void d3d_oracle_requantize(const int32_t* acc, const float* m, const float* bq, 
       float q = rintf(t);  // clamped as a float so the int conversion never overflows
       q = std::fmin(127.f, std::fmax(float(lo), q));
       out[r * cout + c] = int8_t(int(q));
+    }
+  }
+}
+
+// kernel::densify after the memset (trt/spconv/bev_densify_trt.cu:22-35, :160-174): the map is [B, C, Z, Y, X],
+// all zero except out[b, :, z, y, x] = feats[i, :] for every live row i with coordinate (b, z, y, x).  Rows are
+// visited in order, so the last row naming a cell stays (the reference leaves that race open).  Elements are
+// copied as bytes: elemBytes = 4 (float), 2 (half / bf16) or 1 (int8).
+void d3d_oracle_bev_densify(const uint8_t* feats, const int32_t* coors, int32_t numActIn, int C, int elemBytes, int B,
+                            int Z, int Y, int X, uint8_t* out) {
+  const size_t plane = size_t(Z) * Y * X;
+  std::memset(out, 0, size_t(B) * C * plane * elemBytes);
+  for (int32_t i = 0; i < numActIn; i++) {
+    const int32_t* c = coors + size_t(i) * 4;
+    for (int ch = 0; ch < C; ch++) {
+      const size_t at = (size_t(c[0]) * C + ch) * plane + (size_t(c[1]) * Y + c[2]) * X + c[3];
+      std::memcpy(out + at * elemBytes, feats + (size_t(i) * C + ch) * elemBytes, elemBytes);
     }
   }
 }

@@ -13,6 +13,7 @@ import torch
 import deploy3d_amd
 from deploy3d_amd import EngineError, Plugin, TensorDesc
 from deploy3d_amd.plugin import EXPORTS
+from deploy3d_amd.bev_densify import densify_blob
 from deploy3d_amd.spconv_index import index_blob
 from deploy3d_amd.spconv_mm import mm_blob
 
@@ -28,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert getattr(lib, name) is not None
     assert [lib.d3d_op_name(i).decode() for i in range(lib.d3d_num_ops())] == [
-        "SPConvIdx1d", "SPConvIdx2d", "SPConvIdx3d", "SPConvIdx4d", "SPConvMM"]
+        "SPConvIdx1d", "SPConvIdx2d", "SPConvIdx3d", "SPConvIdx4d", "SPConvMM", "BEVDensify"]
 
 
 def test_index_blob_layout_and_round_trip():
@@ -88,12 +89,32 @@ def test_mm_blob_layout_and_round_trip():
     assert len(ext) == len(blob) + 20 and Plugin("SPConvMM", ext).serialize() == ext
 
 
+def test_densify_blob_and_shape_inference():
+    """BEVDensifyPluginParam is one int32 (trt/spconv/bev_densify_trt.cu:43-47; writer bev_densify.py:38);
+    getOutputDimensions gives [B, outChannels, Y, X] (bev_densify_trt.cu:86-97)."""
+    blob = densify_blob(256)
+    assert blob == struct.pack("<i", 256)
+    p = Plugin("BEVDensify", blob)
+    assert p.plugin_type == "BEVDensify" and p.plugin_version == "2.0" and p.num_outputs == 1
+    assert p.serialize() == blob and p.clone().serialize() == blob
+    for dtype, code in ((torch.float32, 0), (torch.float16, 1)):
+        ins = [TensorDesc.of((10000, 128), dtype), TensorDesc.of((10000, 4), torch.int32),
+               TensorDesc.of((1,), torch.int32), TensorDesc.of((2, 0, 2, 128, 128), torch.int32)]
+        outs = p.output_descs(ins)
+        assert [o.shape() for o in outs] == [(2, 256, 128, 128)] and outs[0].dtype == code
+        assert all(p.supports_format(i, ins + outs, 4, 1) for i in range(5))
+        assert p.workspace_size(ins, outs) == 2 * 2 * 128 * 128 * 4
+    bad = [TensorDesc.of((10, 128), torch.int32)] + ins[1:] + outs
+    assert not p.supports_format(0, bad, 4, 1)
+
+
 @pytest.mark.parametrize("name,blob,status", [
     ("SPConvIdx3d", b"\x00" * 10, -2),
     ("SPConvMM", b"\x00" * 5, -2),
     ("SPConvMM", mm_blob((3, 3, 3), 4, 8, 10, True, False, np.zeros(27 * 32, np.float32))[:-40], -2),
     ("SPConvIdx3d", index_blob((0, 3, 3), (1,) * 3, (1,) * 3, (1,) * 3, (0,) * 3, 10, True, False), -2),
-    ("BEVDensify", b"", -4),
+    ("BEVDensify", b"\x00\x00", -2),
+    ("SimpleMeanEncoder", b"", -4),
 ])
 def test_bad_blobs_and_unknown_ops_return_status(name, blob, status):
     with pytest.raises(EngineError) as e:
