@@ -657,12 +657,14 @@ bmMarkCandidates(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const 
   }
 }
 
+constexpr uint32_t kScanGroup = 32;  // workgroups of the scan pass that share one first-level ticket
+
 // One pass over the records: every record gets the count of occupied cells before it INSIDE its chunk of 1024
 // records, every chunk its total; the workgroup that finishes last (a ticket counter, no waiting) turns the chunk
 // totals into exclusive chunk bases and writes numActOut = min(total, maxNumActOut) for strided convolutions.
 __global__ void __launch_bounds__(kRbThreads)
 bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, uint32_t nChunks, uint32_t* ticket,
-       int32_t* numActOut, int32_t maxNumActOut) {
+       uint32_t* groupTickets, int32_t* numActOut, int32_t maxNumActOut) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   __shared__ uint32_t isLast;
   const uint32_t first = blockIdx.x * kRbChunk + threadIdx.x * kRbItems;
@@ -686,7 +688,16 @@ bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, u
     // and only then is the ticket taken.
     uint32_t old = __hip_atomic_exchange(&chunkBase[blockIdx.x], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(old)::"memory");
-    isLast = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nChunks - 1 ? 1u : 0u;
+    // Atomics on one address are performed one after the other (about 18 ns each across the XCDs), so the
+    // tickets are taken in two levels: one counter per kScanGroup workgroups, and only the last of each group
+    // goes on to the counter of the whole grid.
+    const uint32_t group = blockIdx.x / kScanGroup;
+    const uint32_t groupSize = min(kScanGroup, nChunks - group * kScanGroup);
+    const uint32_t nGroups = (nChunks + kScanGroup - 1) / kScanGroup;
+    uint32_t last = 0;
+    if (__hip_atomic_fetch_add(&groupTickets[group], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groupSize - 1)
+      last = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nGroups - 1 ? 1u : 0u;
+    isLast = last;
   }
   __syncthreads();
   if (!isLast) return;
@@ -1157,6 +1168,8 @@ int structureOverride() {
   return 0;
 }
 
+size_t scanGroups(uint32_t nChunks) { return (static_cast<size_t>(nChunks) + kScanGroup - 1) / kScanGroup; }
+
 RbWorkspace planWith(const RbGeom& g, int64_t cap, bool subM, bool blockMap) {
   RbWorkspace w{};
   if (cap < 1) cap = 1;
@@ -1201,8 +1214,9 @@ RbWorkspace planWith(const RbGeom& g, int64_t cap, bool subM, bool blockMap) {
   off = alignUp(off + static_cast<size_t>(g.kVol) * w.pitch * 4);
   w.cnt = off;     // [kVol, nBlocks], directly followed (no gap) by
   off += static_cast<size_t>(g.kVol) * w.nBlocks * 4;
-  w.totals = off;  // [2, kVol] + 2: valid pairs per tap, owned outputs per tap, "rows not in rank order" flag, scan ticket
-  off = alignUp(off + (static_cast<size_t>(g.kVol) * 2 + 2) * 4);
+  w.totals = off;  // [2, kVol] + 2 + groups: valid pairs per tap, owned outputs per tap, "rows not in rank order" flag,
+                   // scan ticket, first-level scan tickets
+  off = alignUp(off + (static_cast<size_t>(g.kVol) * 2 + 2 + scanGroups(w.nChunks)) * 4);
   w.total = off;
   return w;
 }
@@ -1335,7 +1349,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
     hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + (near ? 0 : nIndex / 4) + 1), block, 0,
                        stream, reinterpret_cast<uint4*>(records), static_cast<int64_t>(w.nRecords),
-                       near ? nullptr : index, nIndex, cnt, static_cast<int64_t>(g.kVol) * w.nBlocks + 2 * g.kVol + 2,
+                       near ? nullptr : index, nIndex, cnt,
+                       static_cast<int64_t>(g.kVol) * w.nBlocks + 2 * g.kVol + 2 + static_cast<int64_t>(scanGroups(w.nChunks)),
                        numIndex);
     if (subM) {
       hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
@@ -1351,7 +1366,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       hipLaunchKernelGGL(bmMarkCandidates, perTap, block, 0, stream, g, m, coors, numActIn, cap, records);
     }
     hipLaunchKernelGGL(bmScan, perChunk, block, 0, stream, records, w.nRecords, chunkBase, w.nChunks, scanTicket,
-                       subM ? nullptr : numActOut, maxNumActOut);
+                       scanTicket + 1, subM ? nullptr : numActOut, maxNumActOut);
     if (!near) {  // the near probe launch carries these passes itself
       if (!subM)
         hipLaunchKernelGGL(bmEmitCoords, dim3((w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64)), block, 0, stream,
