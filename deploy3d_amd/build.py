@@ -11,7 +11,7 @@ LIBS = os.path.join(HERE, "libs")
 ENGINE_LIB = os.path.join(LIBS, "libdeploy3d_amd.so")
 SYNTH_LIB = os.path.join(LIBS, "libd3d_synth.so")
 
-ENGINE_SOURCES = ["rulebook.hip", "conv.hip", "densify.hip", "plugin.cpp"]
+ENGINE_SOURCES = ["rulebook.hip", "conv.hip", "densify.hip", "voxelize.hip", "plugin.cpp"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",

@@ -122,6 +122,24 @@ struct DensifyArgs {
   void* workspace;
   size_t workspaceBytes;
 };
+// Points -> voxels with mean features (voxelize.hip).
+struct VoxelizeArgs {
+  const float* feats;       // [numPts, C], x y z first
+  const int32_t* batchIdx;  // [numPts], negative = skip
+  const float* config;      // device float[6]: xMin yMin zMin xSize ySize zSize
+  int64_t numPts;
+  int C;
+  int B, Z, Y, X;
+  int32_t maxNumActOut;
+  float* outFeats;          // [maxNumActOut, C]
+  int32_t* outCoors;        // [maxNumActOut, 4]
+  int32_t* numActOut;       // [1]
+  void* workspace;
+  size_t workspaceBytes;
+};
+size_t voxelizeWorkspaceBytes(int64_t numPts, int64_t maxNumActOut);
+int32_t launchVoxelize(const VoxelizeArgs& a, hipStream_t stream);
+
 size_t densifyWorkspaceBytes(int64_t B, int64_t Z, int64_t Y, int64_t X);
 int32_t launchDensify(const DensifyArgs& a, hipStream_t stream);
 

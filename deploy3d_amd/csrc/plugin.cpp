@@ -899,12 +899,120 @@ struct DensifyPlugin final : d3d_plugin {
   }
 };
 
+// --- SimpleMeanEncoder -------------------------------------------------------
+// Attribute layout: SimpleMeanEncoderPluginParam, one int32 maxNumActOut
+// (trt/voxel_encoder/simple_mean_trt.cu:176-180; written by
+// deploy3d/symfun/ops/voxel_encoder/simple_mean.py:44).
+struct VoxelizePlugin final : d3d_plugin {
+  int32_t maxNumActOut = 0;
+
+  static int32_t parse(const void* data, size_t len, VoxelizePlugin** out) {
+    if (!data || len < 4) {
+      setError("SimpleMeanEncoder: attribute blob of %zu bytes, 4 expected", len);
+      return D3D_ERR_BAD_BLOB;
+    }
+    auto p = std::unique_ptr<VoxelizePlugin>(new VoxelizePlugin());
+    p->type = "SimpleMeanEncoder";
+    std::memcpy(&p->maxNumActOut, data, 4);
+    if (p->maxNumActOut < 0) {
+      setError("SimpleMeanEncoder: maxNumActOut %d", p->maxNumActOut);
+      return D3D_ERR_BAD_BLOB;
+    }
+    p->blob.assign(static_cast<const uint8_t*>(data), static_cast<const uint8_t*>(data) + len);
+    *out = p.release();
+    return D3D_OK;
+  }
+
+  d3d_plugin* clone() const override { return new VoxelizePlugin(*this); }
+  int32_t numOutputs() const override { return 3; }
+  // outFeats [maxNumActOut, C], outCoors [maxNumActOut, 4], numActOut [1] (simple_mean_trt.cu:221-238)
+  int32_t outputDims(int32_t idx, const d3d_tensor_desc* in, int32_t nbIn, d3d_tensor_desc* out) const override {
+    if (idx < 0 || idx > 2 || !out || !in || nbIn < 1 || in[0].nb_dims != 2) return D3D_ERR_BAD_ARG;
+    std::memset(out, 0, sizeof(*out));
+    out->format = D3D_LINEAR;
+    if (idx == 2) {
+      out->nb_dims = 1;
+      out->dims[0] = 1;
+      return D3D_OK;
+    }
+    out->nb_dims = 2;
+    out->dims[0] = maxNumActOut;
+    out->dims[1] = idx == 0 ? in[0].dims[1] : 4;
+    return D3D_OK;
+  }
+  int32_t outputDtype(int32_t idx, const int32_t* inTypes, int32_t nbIn) const override {
+    if (!inTypes || nbIn < 1) return D3D_ERR_BAD_ARG;
+    return idx == 0 ? inTypes[0] : D3D_INT32;  // simple_mean_trt.cu:239-244
+  }
+  // simple_mean_trt.cu:245-258: point features, voxel config and voxel features float; the rest int32
+  int32_t supportsFormat(int32_t pos, const d3d_tensor_desc* io, int32_t nbIn, int32_t nbOut) const override {
+    if (!io || pos < 0 || pos >= nbIn + nbOut || io[pos].format != D3D_LINEAR) return 0;
+    if (pos == 0) return io[0].dtype == D3D_FLOAT;
+    if (pos == 1 || pos == 3 || pos == 5 || pos == 6) return io[pos].dtype == D3D_INT32;
+    return io[pos].dtype == io[0].dtype;
+  }
+  int32_t configure(const d3d_tensor_desc*, int32_t, const d3d_tensor_desc*, int32_t) override { return D3D_OK; }
+  size_t workspaceSize(const d3d_tensor_desc* in, int32_t nbIn) const override {  // simple_mean_trt.cu:273-278
+    if (!in || nbIn < 1 || in[0].nb_dims != 2) return 0;
+    return voxelizeWorkspaceBytes(in[0].dims[0], maxNumActOut);
+  }
+  int32_t enqueue(const d3d_tensor_desc* inDesc, const d3d_tensor_desc* outDesc, const void* const* inputs,
+                  void* const* outputs, void* workspace, size_t workspaceBytes, hipStream_t stream) override {
+    if (!inDesc || !outDesc || !inputs || !outputs) return D3D_ERR_BAD_ARG;
+    if (inDesc[0].nb_dims != 2 || inDesc[0].dims[1] < 3 || inDesc[1].nb_dims != 1 ||
+        inDesc[1].dims[0] != inDesc[0].dims[0] || inDesc[2].nb_dims != 1 || inDesc[2].dims[0] != 6 ||
+        inDesc[3].nb_dims != 5) {
+      setError("SimpleMeanEncoder: expects batchPointFeats [N, C >= 3], batchIndices [N], voxelConfig [6], "
+               "inSpatialShape [B, 0, Z, Y, X]");
+      return D3D_ERR_BAD_ARG;
+    }
+    if (inDesc[0].dtype != D3D_FLOAT || inDesc[2].dtype != D3D_FLOAT || inDesc[1].dtype != D3D_INT32) {
+      setError("SimpleMeanEncoder: point features and voxel config must be float, batch indices int32");
+      return D3D_ERR_UNSUPPORTED;
+    }
+    const int64_t n = inDesc[0].dims[0], C = inDesc[0].dims[1];
+    const int64_t B = inDesc[3].dims[0], Z = inDesc[3].dims[2], Y = inDesc[3].dims[3], X = inDesc[3].dims[4];
+    if (n < 0 || n > 0x7fffffff || C > 4096 || B < 0 || Z < 0 || Y < 0 || X < 0 || B > 0x7fffffff || Z > 0x7fffffff ||
+        Y > 0x7fffffff || X > 0x7fffffff) {
+      setError("SimpleMeanEncoder: tensor extents out of range");
+      return D3D_ERR_BAD_ARG;
+    }
+    if (outDesc[0].nb_dims != 2 || outDesc[0].dims[0] != maxNumActOut || outDesc[0].dims[1] != C ||
+        outDesc[1].nb_dims != 2 || outDesc[1].dims[0] != maxNumActOut || outDesc[1].dims[1] != 4) {
+      setError("SimpleMeanEncoder: outputs must be [maxNumActOut, C] and [maxNumActOut, 4]");
+      return D3D_ERR_BAD_ARG;
+    }
+    if (!outputs[2] || (maxNumActOut > 0 && (!outputs[0] || !outputs[1])) ||
+        (n > 0 && (!inputs[0] || !inputs[1] || !inputs[2]))) {
+      setError("SimpleMeanEncoder: null tensor pointer");
+      return D3D_ERR_BAD_ARG;
+    }
+    VoxelizeArgs a{};
+    a.feats = static_cast<const float*>(inputs[0]);
+    a.batchIdx = static_cast<const int32_t*>(inputs[1]);
+    a.config = static_cast<const float*>(inputs[2]);
+    a.numPts = n;
+    a.C = static_cast<int>(C);
+    a.B = static_cast<int>(B);
+    a.Z = static_cast<int>(Z);
+    a.Y = static_cast<int>(Y);
+    a.X = static_cast<int>(X);
+    a.maxNumActOut = maxNumActOut;
+    a.outFeats = static_cast<float*>(outputs[0]);
+    a.outCoors = static_cast<int32_t*>(outputs[1]);
+    a.numActOut = static_cast<int32_t*>(outputs[2]);
+    a.workspace = workspace;
+    a.workspaceBytes = workspaceBytes;
+    return launchVoxelize(a, stream);
+  }
+};
+
 struct OpEntry {
   const char* name;
-  int nd;  // 0 = SPConvMM, -1 = BEVDensify
+  int nd;  // 0 = SPConvMM, -1 = BEVDensify, -2 = SimpleMeanEncoder
 };
 constexpr OpEntry kOps[] = {{"SPConvIdx1d", 1}, {"SPConvIdx2d", 2}, {"SPConvIdx3d", 3}, {"SPConvIdx4d", 4},
-                            {"SPConvMM", 0},    {"BEVDensify", -1}};
+                            {"SPConvMM", 0},    {"BEVDensify", -1},  {"SimpleMeanEncoder", -2}};
 constexpr const char* kVersion = "2.0";
 
 }  // namespace
@@ -942,7 +1050,13 @@ int32_t d3d_create(const char* name, const char* version, const void* blob, size
   }
   for (const OpEntry& op : kOps) {
     if (std::strcmp(name, op.name) != 0) continue;
-    if (op.nd < 0) {
+    if (op.nd == -2) {
+      VoxelizePlugin* p = nullptr;
+      int32_t rc = VoxelizePlugin::parse(blob, len, &p);
+      *out = p;
+      return rc;
+    }
+    if (op.nd == -1) {
       DensifyPlugin* p = nullptr;
       int32_t rc = DensifyPlugin::parse(blob, len, &p);
       *out = p;

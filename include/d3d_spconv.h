@@ -2,7 +2,8 @@
  *
  * The library exposes the operators of deploy3d's sparse-convolution path (the
  * rulebook builder, the gather-GEMM-scatter, and the sparse-to-dense step that
- * ends the sparse part of a network) as opaque plugin objects with the life cycle TensorRT drives on the
+ * ends the sparse part of a network, and the voxeliser in front of it) as
+ * opaque plugin objects with the life cycle TensorRT drives on the
  * reference's IPluginV2DynamicExt classes: deserialize -> clone -> configure
  * -> workspace size -> enqueue (stream-ordered) -> destroy.  Every function is
  * noexcept, takes plain pointers and sizes, and returns an int32 status.
@@ -11,6 +12,7 @@
  *   "SPConvIdx1d" .. "SPConvIdx4d", version "2.0"   (trt/spconv/index_trt.cu:20-50, :287-290)
  *   "SPConvMM",                     version "2.0"   (trt/spconv/mm_trt.cu:22-37, :239)
  *   "BEVDensify",                   version "2.0"   (trt/spconv/bev_densify_trt.cu:37-47, :209)
+ *   "SimpleMeanEncoder",            version "2.0"   (trt/voxel_encoder/simple_mean_trt.cu:170-180, :346)
  */
 #ifndef D3D_SPCONV_H_
 #define D3D_SPCONV_H_
@@ -64,7 +66,8 @@ typedef struct d3d_plugin d3d_plugin;
  *                  {u32 magic 'D3DX'; u32 version 1; u32 flags (bit0 fused ReLU);
  *                   f32 actScaleIn; f32 actScaleOut} that the reference's parser
  *                  skips as trailing floats.
- *   BEVDensify:    int32 outChannels  (trt/spconv/bev_densify_trt.cu:43-47, :199-204) */
+ *   BEVDensify:    int32 outChannels  (trt/spconv/bev_densify_trt.cu:43-47, :199-204)
+ *   SimpleMeanEncoder: int32 maxNumActOut  (trt/voxel_encoder/simple_mean_trt.cu:176-180, :335-339) */
 int32_t d3d_create(const char* name, const char* version, const void* blob, size_t len, d3d_plugin** out);
 
 /* IPluginV2DynamicExt::clone (index_trt.cu:75-79, mm_trt.cu:75-79): clones share device weights. */
@@ -123,7 +126,14 @@ size_t d3d_workspace_size(const d3d_plugin* p, const d3d_tensor_desc* in, int32_
  *                outputs: 0 outFeatMaps [B, outChannels = C*Z, Y, X], dtype of input 0: zero except
  *                         out[b, c*Z + z, y, x] = inFeats[i, c] for live row i at (b, z, y, x)
  *                workspace: one int32 per grid cell (the reference needs none); rows outside the grid
- *                         are skipped, and of rows naming one cell the highest stays */
+ *                         are skipped, and of rows naming one cell the highest stays
+ * SimpleMeanEncoder (simple_mean_trt.cu:279-311; float features only, as in the reference)
+ *                inputs : 0 batchPointFeats float [N, C >= 3] (x y z first), 1 batchIndices int32 [N]
+ *                         (negative = skip), 2 voxelConfig float [6] on the device (xMin yMin zMin xSize ySize
+ *                         zSize), 3 inSpatialShape (dims [B, 0, Z, Y, X] only; pointer unused)
+ *                outputs: 0 outFeats float [maxNumActOut, C] (mean per voxel; zero past numActOut),
+ *                         1 outCoors int32 [maxNumActOut, 4] (b, z, y, x), 2 numActOut int32 [1]
+ *                         = min(occupied cells, maxNumActOut); voxels in order of first appearance */
 int32_t d3d_enqueue(d3d_plugin* p, const d3d_tensor_desc* in_desc, const d3d_tensor_desc* out_desc,
                     const void* const* inputs, void* const* outputs, void* workspace, size_t workspace_bytes,
                     void* stream);

@@ -146,6 +146,26 @@ def requant_params(s_in, s_w, s_out, bias):
     return m, bq
 
 
+def simple_mean(point_feats, batch_indices, voxel_config, spatial_shape, max_num_act_out):
+    """Voxel means in the reference's (hash-slot) order; spatial_shape = (B, Z, Y, X).
+    Returns (out_feats [max, C] float32, out_coors [max, 4] int32 (-1 past the live rows), num_act_out)."""
+    point_feats = np.ascontiguousarray(point_feats, dtype=np.float32)
+    batch_indices = np.ascontiguousarray(batch_indices, dtype=np.int32)
+    voxel_config = np.ascontiguousarray(voxel_config, dtype=np.float32)
+    n, c = point_feats.shape
+    b, z, y, x = (int(v) for v in spatial_shape)
+    out_feats = np.empty((max_num_act_out, c), dtype=np.float32)
+    out_coors = np.empty((max_num_act_out, 4), dtype=np.int32)
+    num = np.zeros(1, dtype=np.int32)
+    lib().d3d_oracle_simple_mean.restype = ctypes.c_int
+    rc = lib().d3d_oracle_simple_mean(_p(point_feats), _p(batch_indices), _p(voxel_config), ctypes.c_int64(n),
+                                      ctypes.c_int(c), ctypes.c_int(b), ctypes.c_int(z), ctypes.c_int(y), ctypes.c_int(x),
+                                      ctypes.c_int32(int(max_num_act_out)), _p(out_feats), _p(out_coors), _p(num))
+    if rc != 0:
+        raise RuntimeError("oracle simple_mean: hash table full")
+    return out_feats, out_coors, int(num[0])
+
+
 def bev_densify(in_feats, in_coors, num_act_in, spatial_shape):
     """Dense map [B, C*Z, Y, X] of the first num_act_in rows; spatial_shape = (B, Z, Y, X).
     in_feats may be any 1/2/4-byte numpy dtype (fp16 as np.float16, bf16 as its uint16 bits)."""

@@ -21,6 +21,10 @@
 //                  NOT in the reference (trt/spconv/mm_trt.cu:184 accepts fp16
 //                  only): parity unpinned by the reference, pinned only by the
 //                  written rule restated above requantize() below.
+//   simple_mean    torch unique + index_add scatter-mean, the formulation of the
+//                  reference's own test (tests/voxel_encoder/test_simple_mean.py:17-33),
+//                  on that test's two cases; truncation toward zero below the grid's
+//                  minimum, NaN / negative-batch rows, the count under truncation
 //   bev_densify    the dense-indexing ground truth of the reference's own test
 //                  (tests/spconv/test_bev_densify.py:19-23) on its six cases
 //
@@ -373,6 +377,89 @@ void d3d_oracle_bev_densify(const uint8_t* feats, const int32_t* coors, int32_t 
       std::memcpy(out + at * elemBytes, feats + (size_t(i) * C + ch) * elemBytes, elemBytes);
     }
   }
+}
+
+// simpleMeanEncoder (trt/voxel_encoder/simple_mean_trt.cu:26-168), executed serially in point order:
+//   voxelize        (:28-60)  a point counts when all C features are finite, batch >= 0 and its cell
+//                             (b, int((z-zMin)/zSize), int((y-yMin)/ySize), int((x-xMin)/xSize)) - fp32 arithmetic,
+//                             conversion truncating toward zero - is inside the grid; the cell offset goes into a
+//                             linear-probing table of 2*numPts slots (hash32.h:35-72), start slot fmix32(key) % size
+//   inclusive scan  (:147-150) over the slots' occupancy: voxel id = scan - 1, so ids follow SLOT order;
+//                             numActOut = min(occupied slots, maxNumActOut) (:87)
+//   scatterAddFeats (:62-91)  ids below maxNumActOut accumulate feature sums and counts; the first point of a voxel
+//                             writes its coordinate
+//   meanFeats       (:93-101) rows below numActOut are divided by their count
+// outFeats rows from numActOut on are zero (:142); outCoors rows from numActOut on are set to -1 here (the
+// reference leaves them unwritten).  Returns 0, or -1 on a full table (cannot happen at load factor 1/2).
+int d3d_oracle_simple_mean(const float* feats, const int32_t* batchIdx, const float* config, int64_t numPts, int C,
+                           int B, int Z, int Y, int X, int32_t maxNumActOut, float* outFeats, int32_t* outCoors,
+                           int32_t* numActOut) {
+  const int64_t size = numPts * 2;
+  std::vector<int64_t> key(size > 0 ? size : 1, -1);
+  std::vector<int64_t> slotOf(numPts > 0 ? numPts : 1, -1);
+  // float -> int32 as the device conversion does it: toward zero, saturating, NaN -> 0
+  auto toInt = [](float v) -> int64_t {
+    if (std::isnan(v)) return 0;
+    if (v >= 2147483648.f) return 2147483647LL;
+    if (v <= -2147483648.f) return -2147483648LL;
+    return int64_t(int32_t(v));
+  };
+  for (int64_t i = 0; i < numPts; i++) {
+    const float* f = feats + i * C;
+    bool ok = true;
+    for (int c = 0; c < C; c++) ok = ok && std::isfinite(f[c]);
+    if (!ok) continue;
+    const int64_t b = batchIdx[i];
+    if (b < 0) continue;
+    const int64_t x = toInt((f[0] - config[0]) / config[3]);
+    const int64_t y = toInt((f[1] - config[1]) / config[4]);
+    const int64_t z = toInt((f[2] - config[2]) / config[5]);
+    if (b > B - 1 || z < 0 || z > Z - 1 || y < 0 || y > Y - 1 || x < 0 || x > X - 1) continue;
+    const int64_t off = ((b * Z + z) * Y + y) * X + x;
+    int64_t slot = int64_t(fmix32(uint32_t(off)) % uint64_t(size));
+    int64_t tries = 0;
+    for (; tries < size; tries++) {
+      if (key[slot] == -1 || key[slot] == off) {
+        key[slot] = off;
+        slotOf[i] = slot;
+        break;
+      }
+      slot = (slot + 1) % size;
+    }
+    if (tries == size) return -1;
+  }
+  std::vector<int32_t> scan(size > 0 ? size : 1, 0);
+  int32_t run = 0;
+  for (int64_t s = 0; s < size; s++) {
+    run += key[s] != -1 ? 1 : 0;
+    scan[s] = run;
+  }
+  *numActOut = run > maxNumActOut ? maxNumActOut : run;
+  std::fill(outFeats, outFeats + int64_t(maxNumActOut) * C, 0.f);
+  std::fill(outCoors, outCoors + int64_t(maxNumActOut) * 4, -1);
+  std::vector<int32_t> count(maxNumActOut > 0 ? maxNumActOut : 1, 0);
+  for (int64_t i = 0; i < numPts; i++) {
+    const int64_t slot = slotOf[i];
+    if (slot < 0) continue;
+    const int32_t id = scan[slot] - 1;
+    if (id >= maxNumActOut) continue;
+    const int32_t firstOne = count[id]++;
+    for (int c = 0; c < C; c++) outFeats[int64_t(id) * C + c] += feats[i * C + c];
+    if (firstOne == 0) {
+      int64_t off = key[slot];
+      int32_t* row = outCoors + int64_t(id) * 4;
+      row[3] = int32_t(off % X);
+      off /= X;
+      row[2] = int32_t(off % Y);
+      off /= Y;
+      row[1] = int32_t(off % Z);
+      off /= Z;
+      row[0] = int32_t(off);
+    }
+  }
+  for (int32_t r = 0; r < *numActOut; r++)
+    for (int c = 0; c < C; c++) outFeats[int64_t(r) * C + c] = outFeats[int64_t(r) * C + c] / float(count[r]);
+  return 0;
 }
 
 }  // extern "C"

@@ -14,6 +14,7 @@ import deploy3d_amd
 from deploy3d_amd import EngineError, Plugin, TensorDesc
 from deploy3d_amd.plugin import EXPORTS
 from deploy3d_amd.bev_densify import densify_blob
+from deploy3d_amd.simple_mean import simple_mean_blob
 from deploy3d_amd.spconv_index import index_blob
 from deploy3d_amd.spconv_mm import mm_blob
 
@@ -29,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert getattr(lib, name) is not None
     assert [lib.d3d_op_name(i).decode() for i in range(lib.d3d_num_ops())] == [
-        "SPConvIdx1d", "SPConvIdx2d", "SPConvIdx3d", "SPConvIdx4d", "SPConvMM", "BEVDensify"]
+        "SPConvIdx1d", "SPConvIdx2d", "SPConvIdx3d", "SPConvIdx4d", "SPConvMM", "BEVDensify", "SimpleMeanEncoder"]
 
 
 def test_index_blob_layout_and_round_trip():
@@ -108,13 +109,33 @@ def test_densify_blob_and_shape_inference():
     assert not p.supports_format(0, bad, 4, 1)
 
 
+def test_simple_mean_blob_and_shape_inference():
+    """SimpleMeanEncoderPluginParam is one int32 (trt/voxel_encoder/simple_mean_trt.cu:176-180; writer
+    simple_mean.py:44); outputs [max, C] float, [max, 4] int32, [1] int32 (simple_mean_trt.cu:221-244)."""
+    blob = simple_mean_blob(30000)
+    assert blob == struct.pack("<i", 30000)
+    p = Plugin("SimpleMeanEncoder", blob)
+    assert p.plugin_type == "SimpleMeanEncoder" and p.plugin_version == "2.0" and p.num_outputs == 3
+    assert p.serialize() == blob and p.clone().serialize() == blob
+    ins = [TensorDesc.of((200000, 5), torch.float32), TensorDesc.of((200000,), torch.int32),
+           TensorDesc.of((6,), torch.float32), TensorDesc.of((2, 0, 41, 1536, 1536), torch.int32)]
+    outs = p.output_descs(ins)
+    assert [o.shape() for o in outs] == [(30000, 5), (30000, 4), (1,)]
+    assert [o.dtype for o in outs] == [0, 3, 3]
+    assert all(p.supports_format(i, ins + outs, 4, 3) for i in range(7))
+    assert p.workspace_size(ins, outs) >= 2 * 200000 * 8
+    half = [TensorDesc.of((200000, 5), torch.float16)] + ins[1:] + outs
+    assert not p.supports_format(0, half, 4, 3)
+
+
 @pytest.mark.parametrize("name,blob,status", [
     ("SPConvIdx3d", b"\x00" * 10, -2),
     ("SPConvMM", b"\x00" * 5, -2),
     ("SPConvMM", mm_blob((3, 3, 3), 4, 8, 10, True, False, np.zeros(27 * 32, np.float32))[:-40], -2),
     ("SPConvIdx3d", index_blob((0, 3, 3), (1,) * 3, (1,) * 3, (1,) * 3, (0,) * 3, 10, True, False), -2),
     ("BEVDensify", b"\x00\x00", -2),
-    ("SimpleMeanEncoder", b"", -4),
+    ("SimpleMeanEncoder", b"\x01", -2),
+    ("CylinderEncoder", b"", -4),
 ])
 def test_bad_blobs_and_unknown_ops_return_status(name, blob, status):
     with pytest.raises(EngineError) as e:
