@@ -730,12 +730,8 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
           }
         }
       }
-      if (a + NS < steps) {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot has been read before it is refilled
-        issueRows(a + NS, slot);
-      }
-      // every weight fragment of the step is requested before the first MFMA, so the MFMAs start as the
-      // fragments arrive instead of paying the LDS latency once per fragment pair
+      // every fragment of the step - rows, then weights - is requested before the first MFMA, so the LDS pipe
+      // works from the first cycle of the step and the MFMAs start as the fragments arrive
       const F* wTap = reinterpret_cast<const F*>(wLds + (RESIDENT ? a : wbuf) * WCH);
       F wts[KK][NT];
 #pragma unroll
@@ -753,6 +749,12 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
             } else {
               acc[m][n] = Mfma<T>::k16(wts[kk][n], rows[m][kk], acc[m][n]);
             }
+          }
+          if (kk == 0 && n == 0 && a + NS < steps) {
+            // LDS reads return in order: once all but the last KK*NT-1 (weight fragments) are back, every row
+            // fragment of the slot has been read and the slot may be refilled
+            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(KK * NT - 1) : "memory");
+            issueRows(a + NS, slot);
           }
         }
       }
