@@ -711,25 +711,34 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
 #pragma unroll
       for (int n = 0; n < NT; ++n) acc[m][n] = Acc{0, 0, 0, 0};
 
-    int slot = 0, wbuf = 0;
-    for (int a = 0; a < steps; ++a) {
-      const bool steady = a + NS + 3 < steps;
-      if (steady) issueIndex(a + NS + 3);
-      if (!RESIDENT && a + 2 < steps) issueWeights(a + 2);
-      F rows[MT][KK];
+    // Row fragments of a step are read from LDS at the end of the step before (its rows have landed by then and
+    // belong to this wavefront alone), so those reads overlap the tail of the MFMAs and the barrier instead of
+    // standing in front of the next step's MFMAs.
+    F rows[MT][KK], rowsNext[MT][KK];
+    auto readRows = [&](F (&dst)[MT][KK], int fromSlot) __attribute__((always_inline)) {
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         const int n = m * 16 + r16;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
           if constexpr (WIDE) {
-            rows[m][kk] = stage[slot * SLOTS + n * CH + ((kk * 4 + kgrp) ^ stageSwizzle<CH>(n))];
+            dst[m][kk] = stage[fromSlot * SLOTS + n * CH + ((kk * 4 + kgrp) ^ stageSwizzle<CH>(n))];
           } else {
-            const u32x2* s2 = reinterpret_cast<const u32x2*>(stage + slot * SLOTS + n * CH + ((kgrp >> 1) ^ stageSwizzle<CH>(n)));
-            rows[m][kk] = s2[kgrp & 1];
+            const u32x2* s2 = reinterpret_cast<const u32x2*>(stage + fromSlot * SLOTS + n * CH + ((kgrp >> 1) ^ stageSwizzle<CH>(n)));
+            dst[m][kk] = s2[kgrp & 1];
           }
         }
       }
+    };
+    readRows(rows, 0);
+
+    int slot = 0, wbuf = 0;
+    // one step; `cur` holds its row fragments, `nxt` receives those of the step after (the caller swaps the two
+    // from step to step, so no fragment is ever copied)
+    auto step = [&](int a, F (&cur)[MT][KK], F (&nxt)[MT][KK]) __attribute__((always_inline)) {
+      const bool steady = a + NS + 3 < steps;
+      if (steady) issueIndex(a + NS + 3);
+      if (!RESIDENT && a + 2 < steps) issueWeights(a + 2);
       // every fragment of the step - rows, then weights - is requested before the first MFMA, so the LDS pipe
       // works from the first cycle of the step and the MFMAs start as the fragments arrive
       const F* wTap = reinterpret_cast<const F*>(wLds + (RESIDENT ? a : wbuf) * WCH);
@@ -745,15 +754,13 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
 #pragma unroll
           for (int m = 0; m < MT; ++m) {
             if constexpr (WIDE) {
-              acc[m][n] = Mfma<T>::k32(wts[kk][n], rows[m][kk], acc[m][n]);
+              acc[m][n] = Mfma<T>::k32(wts[kk][n], cur[m][kk], acc[m][n]);
             } else {
-              acc[m][n] = Mfma<T>::k16(wts[kk][n], rows[m][kk], acc[m][n]);
+              acc[m][n] = Mfma<T>::k16(wts[kk][n], cur[m][kk], acc[m][n]);
             }
           }
           if (kk == 0 && n == 0 && a + NS < steps) {
-            // LDS reads return in order: once all but the last KK*NT-1 (weight fragments) are back, every row
-            // fragment of the slot has been read and the slot may be refilled
-            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(KK * NT - 1) : "memory");
+            // the row fragments of this slot were read a step ago and have just been multiplied: refill it
             issueRows(a + NS, slot);
           }
         }
@@ -787,10 +794,15 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
         else if (allowed >= GL) waitVmcnt<cmin(GL, 63)>();
         else waitVmcnt<0>();
       }
-      // a bare barrier: __syncthreads() would also drain every load in flight, i.e. the whole prefetch
-      if (!RESIDENT) __builtin_amdgcn_s_barrier();
       slot = slot + 1 == NS ? 0 : slot + 1;
       wbuf = wbuf + 1 == NWB ? 0 : wbuf + 1;
+      if (a + 1 < steps) readRows(nxt, slot);
+      // a bare barrier: __syncthreads() would also drain every load in flight, i.e. the whole prefetch
+      if (!RESIDENT) __builtin_amdgcn_s_barrier();
+    };
+    for (int a = 0; a < steps; a += 2) {
+      step(a, rows, rowsNext);
+      if (a + 1 < steps) step(a + 1, rowsNext, rows);
     }
 
     // epilogue: bias, ReLU, rounding; rows leave through the stage area as contiguous lines
