@@ -454,7 +454,7 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
           const uint32_t* __restrict__ staging, const uint32_t* __restrict__ cnt, uint32_t nBlocks,
           const uint32_t* __restrict__ totals, int32_t* __restrict__ gather, int32_t* __restrict__ scatter,
           int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* __restrict__ nbr, int64_t nbrRows,
-          const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled) {
+          const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int mirror) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int tap = blockIdx.y;
   const uint32_t b = blockIdx.x;
@@ -464,37 +464,59 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
     *numIndex = static_cast<int32_t>(end);
   }
   const int n = liveCount(numActIn, cap);
-  if (static_cast<int64_t>(b) * kRbChunk >= n) return;           // workgroup-uniform
-  if (cnt[static_cast<size_t>(tap) * nBlocks + b] == 0) return;  // workgroup-uniform
+  const int64_t first = static_cast<int64_t>(b) * kRbChunk + threadIdx.x * kRbItems;
+  // Mirror mode (SubM with "same" padding): the pair (tap, in i -> out o) has the twin (kVol-1-tap, in o -> out i),
+  // so row i of the neighbour table under the mirrored tap is simply o - this thread's own staging entry.  The
+  // table is then written here in whole coalesced rows, -1 included: no fill pass, no scatter.
+  int32_t* nbrRow = (mirror && nbr) ? nbr + static_cast<int64_t>(kVol - 1 - tap) * nbrRows : nullptr;
+  auto mirrorStore = [&](const uint32_t (&o)[kRbItems]) {
+    if (!nbrRow) return;
+    if (first + kRbItems <= nbrRows && ((reinterpret_cast<uintptr_t>(nbrRow + first) & 15) == 0)) {
+      *reinterpret_cast<uint4*>(nbrRow + first) = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < kRbItems; ++j)
+        if (first + j < nbrRows) nbrRow[first + j] = static_cast<int32_t>(o[j]);
+    }
+  };
+  const uint32_t none4[kRbItems] = {kNone, kNone, kNone, kNone};
+  if (static_cast<int64_t>(b) * kRbChunk >= n || cnt[static_cast<size_t>(tap) * nBlocks + b] == 0) {  // workgroup-uniform
+    mirrorStore(none4);
+    return;
+  }
 
   uint32_t before = 0;
   for (uint32_t q = threadIdx.x; q < b; q += blockDim.x) before += cnt[static_cast<size_t>(tap) * nBlocks + q];
   uint32_t pos = blockSum(before, scratch);
   for (int t = 0; t < tap; ++t) pos += (totals[t] + (kSegment - 1)) & ~static_cast<uint32_t>(kSegment - 1);
 
-  const int64_t first = static_cast<int64_t>(b) * kRbChunk + threadIdx.x * kRbItems;
   uint4 s4 = make_uint4(kNone, kNone, kNone, kNone);
   if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<size_t>(tap) * pitch + first);
   uint32_t v[kRbItems] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+  for (int j = 0; j < kRbItems; ++j)
+    if (first + j >= n) v[j] = kNone;
   if (perm && *permShuffled) {  // block-map SubM: the probe stored ranks; rows are perm[rank]
 #pragma unroll
     for (int j = 0; j < kRbItems; ++j)
-      if (first + j < n && v[j] != kNone) v[j] = perm[v[j]];
+      if (v[j] != kNone) v[j] = perm[v[j]];
   }
+  mirrorStore(v);
   uint32_t mine = 0;
 #pragma unroll
-  for (int j = 0; j < kRbItems; ++j) mine += (first + j < n && v[j] != kNone);
+  for (int j = 0; j < kRbItems; ++j) mine += (v[j] != kNone);
   uint32_t total;
   uint32_t at = pos + blockExclusiveScan(mine, scratch, &total);
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
-    if (first + j < n && v[j] != kNone) {
+    if (v[j] != kNone) {
       gather[at] = static_cast<int32_t>(first + j);
       scatter[at] = static_cast<int32_t>(v[j]);
       tapRow[at] = tap;
       ++at;
       // the same pair in output-major form, for the convolution: nbr[tap][output row] = input row
-      if (nbr && v[j] < static_cast<uint64_t>(nbrRows)) nbr[static_cast<int64_t>(tap) * nbrRows + v[j]] = static_cast<int32_t>(first + j);
+      if (nbr && !mirror && v[j] < static_cast<uint64_t>(nbrRows))
+        nbr[static_cast<int64_t>(tap) * nbrRows + v[j]] = static_cast<int32_t>(first + j);
     }
   }
 }
@@ -1328,7 +1350,16 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     return dim3(static_cast<unsigned>(blocks < 1 ? 1 : blocks));
   };
 
-  bool nbrFilled = false;
+  // SubM with stride 1 and padding (k-1)*d/2 in every dim: pairs come in mirrored twins, and the compaction
+  // writes the neighbour table row by row (see rbCompact).  D3D_RULEBOOK_MIRROR=0 switches it off (tests).
+  bool mirror = subM && nbrOut && nbrRows == cap && !g.transpose;
+  for (int dim = 0; dim < kMaxSpatial; ++dim)
+    if (g.s[dim] != 1 || 2 * g.p[dim] != (g.k[dim] - 1) * g.d[dim]) mirror = false;
+  {
+    const char* e = std::getenv("D3D_RULEBOOK_MIRROR");
+    if (e && e[0] == '0') mirror = false;
+  }
+  bool nbrFilled = mirror;
   const uint32_t* compactPerm = nullptr;      // block-map SubM: staging holds ranks, rows = perm[rank] when shuffled
   const uint32_t* compactPermFlag = nullptr;
   if (w.blockMap) {
@@ -1380,7 +1411,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       const uint32_t quads = probeBlocks;
       const uint32_t extra = subM ? probeBlocks : (w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64);
       const dim3 fused(quads * 2 + extra);
-      int32_t* fillB = (nbrOut && nbrRows > 0) ? nbrOut : nullptr;
+      int32_t* fillB = (nbrOut && nbrRows > 0 && !mirror) ? nbrOut : nullptr;
       const int64_t nFillB = fillB ? static_cast<int64_t>(g.kVol) * nbrRows : 0;
       nbrFilled = true;
 #define D3D_LAUNCH_PROBE_NEAR(SUBM, KSEL)                                                                          \
@@ -1440,7 +1471,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
                        static_cast<int64_t>(g.kVol) * nbrRows);
   hipLaunchKernelGGL(rbCompact, perTap, block, 0, stream, numActIn, cap, w.pitch, g.kVol, staging, cnt, w.nBlocks,
                      totals, index, index + rowLen, index + 2 * rowLen, numIndex, nbrRows > 0 ? nbrOut : nullptr, nbrRows,
-                     compactPerm, compactPermFlag);
+                     compactPerm, compactPermFlag, mirror ? 1 : 0);
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;
 }

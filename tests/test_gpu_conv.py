@@ -102,6 +102,26 @@ def test_kernel_shapes(engine, ksize, padding):
     run_case(2500, (10, 36, 30), ksize, (1, 1, 1), padding, 32, 64, "float16", True)
 
 
+def test_mirrored_neighbour_table(engine, monkeypatch):
+    """SubM with 'same' padding: the compaction writes the output-major table from the mirrored twin of every pair
+    instead of scattering; D3D_RULEBOOK_MIRROR=0 selects the scatter.  Both must give the same features bit for bit,
+    for shuffled rows and for rows in rank order; a SubM geometry without the symmetry (padding (1, 1, 0)) takes the
+    scatter by itself and must still match the oracle."""
+    from deploy3d_amd.plugin import clear_cache
+    for ksize, padding in (((3, 3, 3), (1, 1, 1)), ((3, 1, 3), (1, 0, 1)), ((5, 5, 5), (2, 2, 2))):
+        monkeypatch.delenv("D3D_RULEBOOK_MIRROR", raising=False)
+        clear_cache()
+        a, _ = run_case(3000, (10, 36, 30), ksize, (1, 1, 1), padding, 32, 64, "float16", True, seed=5)
+        monkeypatch.setenv("D3D_RULEBOOK_MIRROR", "0")
+        clear_cache()
+        b, _ = run_case(3000, (10, 36, 30), ksize, (1, 1, 1), padding, 32, 64, "float16", True, seed=5)
+        assert np.array_equal(a, b)
+    monkeypatch.delenv("D3D_RULEBOOK_MIRROR", raising=False)
+    clear_cache()
+    run_case(3000, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 0), 32, 64, "float16", True, seed=6)
+    run_case(3000, (10, 36, 30), (3, 3, 2), (1, 1, 1), (1, 1, 0), 16, 32, "float16", True, seed=7)
+
+
 @pytest.mark.parametrize("tile_rows", [128, 256, 512])
 @pytest.mark.parametrize("cin,cout", [(32, 64), (64, 64), (64, 128), (128, 128)])
 def test_mfma_tile_sizes(engine, monkeypatch, tile_rows, cin, cout):
