@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the roofline kernel at the default 120 000 voxels, from two `rocprofv3 --pmc` runs of this
 # script (FETCH_SIZE 33873, WRITE_SIZE 32768 per dispatch), each scaled by what the same counter read for the
 # 256 MiB copy of --pmc-copy-mib (FETCH_SIZE reads half the copied KiB: factor 2.0; WRITE_SIZE factor 1.0).
-MEASURED_TRAFFIC_BYTES = {("conv3", 120000): int((33873 * 2.0 + 32768 * 1.0) * 1024)}
+MEASURED_TRAFFIC_BYTES = {("conv3", 120000): int((33911 * 2.0 + 32768 * 1.0) * 1024)}
 
 
 def cpu_baseline(cfg, threads):
