@@ -602,7 +602,6 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
            int relu, int tileBlocks) {
   constexpr int THREADS = 64 * WAVES;
   constexpr int ES = static_cast<int>(sizeof(T));              // 2: fp16 / bf16, 1: int8
-  constexpr int EPC = 16 / ES;                                 // elements per 16-byte chunk
   constexpr int CS = CIN / KS;                                 // input channels per step (a tap takes KS steps)
   constexpr int CH = CS * ES / 16;                             // 16-byte chunks of a row staged per step
   constexpr bool WIDE = CS * ES >= 64;                         // 16-byte operand fragments (else 8-byte)

@@ -184,3 +184,22 @@ def test_unsupported_dtype_returns_minus_one(engine):
         spconv_mm(x, one, one, idx, one, (3, 3, 3), 16, 16, 128, True, False, np.zeros(27 * 16 * 16, np.float32))
     if isinstance(e.value, EngineError):
         assert e.value.status == -1
+
+
+def test_random_layers(engine):
+    """Seeded sweep over random layers: channel counts on and off the MFMA shapes, all storage types, SubM and
+    strided, kernel shapes, bias / ReLU / inverse, live rows short of the capacity - each against the fp64 oracle."""
+    rng = np.random.default_rng(977)
+    channels = [1, 3, 5, 8, 16, 20, 32, 48, 64, 96, 128]
+    kernels = [((3, 3, 3), (1, 1, 1)), ((3, 1, 3), (1, 0, 1)), ((1, 3, 3), (0, 1, 1)), ((1, 1, 1), (0, 0, 0)),
+               ((2, 2, 2), (0, 0, 0)), ((3, 3, 1), (1, 1, 0))]
+    for i in range(30):
+        cin, cout = (int(rng.choice(channels)) for _ in range(2))
+        dtype = ("float16", "bfloat16", "float32")[int(rng.integers(0, 3))]
+        ksize, padding = kernels[int(rng.integers(0, len(kernels)))]
+        subm = bool(rng.integers(0, 2))
+        stride = (1, 1, 1) if subm else tuple(int(rng.integers(1, 3)) for _ in range(3))
+        inverse = (not subm) and bool(rng.integers(0, 4) == 0)
+        run_case(int(rng.integers(200, 2500)), (10, 30, 28), ksize, stride, padding, cin, cout, dtype, subm,
+                 with_bias=bool(rng.integers(0, 2)), relu=bool(rng.integers(0, 2)), inverse=inverse, seed=100 + i,
+                 cap_extra=int(rng.integers(0, 3)) * 37)

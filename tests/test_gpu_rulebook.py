@@ -170,3 +170,59 @@ def test_single_voxel_and_full_block(engine):
     expected = sum((4 - abs(dz)) * (5 - abs(dy)) * (6 - abs(dx)) for dz in (-1, 0, 1) for dy in (-1, 0, 1)
                    for dx in (-1, 0, 1))
     assert live.sum() == expected
+
+
+def _random_geometry(rng):
+    """A random but valid layer: 1 to 4 dims, kernel 1..5, stride 1..3, padding 0..2, dilation 1..2."""
+    nd = int(rng.integers(1, 5))
+    budget = 4096 if nd < 4 else 1500            # cells of the grid: keeps the oracle and the brute force quick
+    side = max(3, int(round(budget ** (1.0 / nd))))
+    grid = tuple(int(rng.integers(max(3, side // 2), side + 3)) for _ in range(nd))
+    ksize = tuple(int(rng.integers(1, 6 if nd < 3 else 4)) for _ in range(nd))
+    dilation = tuple(int(rng.integers(1, 3)) for _ in range(nd))
+    stride = tuple(int(rng.integers(1, 4)) for _ in range(nd))
+    padding = tuple(int(rng.integers(0, 3)) for _ in range(nd))
+    batch = int(rng.integers(1, 4))
+    return nd, grid, ksize, stride, padding, dilation, batch
+
+
+def test_random_geometries(engine):
+    """Seeded sweep over random layer geometries (all three kinds: SubM, strided, transposed), each compared with
+    the oracle: SubM bit for bit, the others after the canonical sort."""
+    rng = np.random.default_rng(20240611)
+    done = 0
+    while done < 36:
+        nd, grid, ksize, stride, padding, dilation, batch = _random_geometry(rng)
+        kind = ("subm", "conv", "transpose")[done % 3]
+        cells = batch * int(np.prod(grid))
+        n = int(rng.integers(1, max(2, min(1500, cells // 2))))
+        coords = random_cloud(rng, n, grid, batch)
+        n = len(coords)
+        kvol = int(np.prod(ksize))
+        if kind == "subm":
+            stride1 = (1,) * nd
+            ref = oracle.rulebook(coords, n, (batch,) + grid, ksize, stride1, padding, dilation, n, True)
+            got = gpu_rulebook(coords, n, grid, batch, ksize, stride1, padding, dilation, n, True)
+            assert got["num_index"] == ref["num_index"], (grid, ksize, padding, dilation)
+            np.testing.assert_array_equal(got["index"], ref["index"])
+        else:
+            transpose = kind == "transpose"
+            out_pad = tuple(int(rng.integers(0, s)) for s in stride) if transpose else None
+            out_grid = oracle.out_shape(grid, ksize, stride, padding, dilation, out_pad, transpose)
+            if min(out_grid) < 1 or batch * int(np.prod(out_grid)) > 200000:
+                continue
+            max_out = min(n * kvol, batch * int(np.prod(out_grid)))
+            ref = oracle.rulebook(coords, n, [batch] + out_grid, ksize, stride, padding, dilation, max_out, False,
+                                  transpose)
+            got = gpu_rulebook(coords, n, grid, batch, ksize, stride, padding, dilation, max_out, False, transpose,
+                               out_padding=out_pad)
+            where = (kind, grid, ksize, stride, padding, dilation, out_pad)
+            assert got["out_grid"] == out_grid, where
+            assert got["num_act_out"] == ref["num_act_out"], where
+            assert got["num_index"] == ref["num_index"], where
+            c_ref, t_ref = oracle.canonical(ref["index"], ref["num_index"], ref["out_coors"], ref["num_act_out"])
+            c_got, t_got = oracle.canonical(got["index"], got["num_index"], got["out_coors"], got["num_act_out"])
+            np.testing.assert_array_equal(c_got, c_ref, err_msg=str(where))
+            np.testing.assert_array_equal(t_got, t_ref, err_msg=str(where))
+        check_index_structure(got["index"], got["num_index"], kvol, n)
+        done += 1
