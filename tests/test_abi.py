@@ -147,3 +147,19 @@ def test_wrong_version_is_unknown_op():
     with pytest.raises(EngineError) as e:
         Plugin("SPConvMM", mm_blob((1, 1, 1), 1, 1, 1, True, False, np.zeros(1, np.float32)), version="1.0")
     assert e.value.status == -4
+
+
+def test_header_is_c_and_a_c_client_works(tmp_path):
+    """include/d3d_spconv.h compiles as C99 and a plain C program drives the library through it (no GPU work)."""
+    import shutil
+    import subprocess
+    from deploy3d_amd.build import ENGINE_LIB
+    gcc = shutil.which("gcc")
+    assert gcc, "gcc is part of the image"
+    exe = tmp_path / "abi_check"
+    src = os.path.join(ROOT, "tests", "abi_c", "abi_check.c")
+    subprocess.check_call([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"),
+                           src, "-o", str(exe), "-ldl"])
+    deploy3d_amd.load_library()  # builds the library if it is not there yet
+    res = subprocess.run([str(exe), ENGINE_LIB], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert res.returncode == 0 and "abi_check ok" in res.stdout, res.stdout
