@@ -730,6 +730,7 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
       }
     };
     readRows(rows, 0);
+    asm volatile("" ::: "memory");
 
     int slot = 0, wbuf = 0;
     // one step; `cur` holds its row fragments, `nxt` receives those of the step after (the caller swaps the two
@@ -796,6 +797,10 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
       slot = slot + 1 == NS ? 0 : slot + 1;
       wbuf = wbuf + 1 == NWB ? 0 : wbuf + 1;
       if (a + 1 < steps) readRows(nxt, slot);
+      // Compiler fence: the weight-fragment reads of the next step stay behind these reads in program order.  LDS
+      // reads return in order, so the first MFMA of a step (which waits for a weight fragment) then implies that
+      // every row fragment of the slot has left LDS, and the slot may be refilled right after it.
+      asm volatile("" ::: "memory");
       // a bare barrier: __syncthreads() would also drain every load in flight, i.e. the whole prefetch
       if (!RESIDENT) __builtin_amdgcn_s_barrier();
     };
