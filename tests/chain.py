@@ -45,6 +45,7 @@ def oracle_chain(cfg, threads=1, acc="f64"):
                 rb["out_coors"] = rb["out_coors"][:rb["num_act_out"]].copy()
                 rb["out_grid"] = og
             rb["pairs"] = int((rb["index"][2, :rb["num_index"]] >= 0).sum())
+            rb["in_coors"] = x["coords"]
             rulebooks[spec["key"]] = rb
         n_out = rb["num_act_out"]
         y = oracle.conv(x["feats"], round_to(w, dtype), round_to(b, dtype), rb["index"], rb["num_index"], n_out,
@@ -72,6 +73,25 @@ def oracle_chain_int8(cfg, rulebook_chain):
         cur = oracle.requantize(acc, m, bq, bool(spec.get("relu")))
         outs[spec["name"]] = cur
     return outs
+
+
+def canonical_pairs(index, num_index, in_coors, num_act_in, out_coors, num_act_out):
+    """Canonical form of a rulebook inside a chain, where the row numbering of the INPUT voxels is as arbitrary as
+    that of the outputs (they are the outputs of an earlier strided layer): both sides are relabelled by the rank
+    of their coordinate, then the triples (tap, gather, scatter) are sorted.  Returns (sorted output coordinates,
+    triples) as int64 arrays."""
+    def ranks(coords, n):
+        c = np.asarray(coords)[:n].astype(np.int64)
+        order = np.lexsort(c.T[::-1])
+        r = np.empty(n, dtype=np.int64)
+        r[order] = np.arange(n)
+        return c[order], r
+    _, rin = ranks(in_coors, num_act_in)
+    cout, rout = ranks(out_coors, num_act_out)
+    g, s, t = (np.asarray(index)[r, :num_index].astype(np.int64) for r in range(3))
+    live = t >= 0
+    tri = np.stack([t[live], rin[g[live]], rout[s[live]]], axis=1)
+    return cout, tri[np.lexsort((tri[:, 2], tri[:, 1], tri[:, 0]))]
 
 
 def sort_rows(coords, feats):

@@ -45,11 +45,19 @@ def compare_chain(cfg, net, ref, tol_scale=1.0):
 
 
 def compare_rulebooks(cfg, net, ref):
+    """Every rulebook of the pass against the oracle's, bit for bit in canonical form: output coordinates sorted,
+    gather and scatter ids relabelled by the rank of their coordinate, triples (tap, gather, scatter) sorted."""
     for key, rb in net.rulebooks.items():
         name = next(s["name"] for s in cfg["layers"] if s["key"] == key)
         n_out = int(rb.num_act_out.item())
         ni = int(rb.num_index.item())
-        c_got, t_got = oracle.canonical(rb.index.cpu().numpy(), ni, rb.out_coors.cpu().numpy(), n_out)
+        c_got, t_got = chain.canonical_pairs(rb.index.cpu().numpy(), ni, rb.in_coors.cpu().numpy(),
+                                             int(rb.num_act_in.item()), rb.out_coors.cpu().numpy(), n_out)
+        orb = ref["_rulebooks"][key]
+        c_ref, t_ref = chain.canonical_pairs(orb["index"], orb["num_index"], orb["in_coors"], len(orb["in_coors"]),
+                                             orb["out_coors"], orb["num_act_out"])
+        np.testing.assert_array_equal(c_got, c_ref, err_msg=key)
+        np.testing.assert_array_equal(t_got, t_ref, err_msg=key)
         assert len(t_got) == ref[name]["pairs"], key
         assert ni % 128 == 0
 
@@ -240,3 +248,99 @@ def test_config5_full_size_runs(engine):
     live = rb.index[2, :ni] >= 0
     cnt = torch.bincount(rb.index[2, :ni][live], minlength=9)
     assert bool((cnt == cnt.flip(0)).all()) and int(cnt[4]) == 250000
+
+
+def _sampled_rows_reference(rb, rows, in_feats, w_tap_major, n_in):
+    """For the output rows in ``rows``: the pairs that reach them, taken from the index tensor the GPU itself emitted
+    (its rulebooks are checked against the oracle elsewhere), as (row position, tap, input row) arrays."""
+    ni = int(rb.num_index.item())
+    g, s, t = (rb.index[r, :ni] for r in range(3))
+    pos = torch.full((int(rb.out_coors.shape[0]) + 1,), -1, dtype=torch.int64, device="cuda")
+    pos[rows] = torch.arange(len(rows), device="cuda")
+    live = t >= 0
+    sel = live & (pos[s.clamp(min=0).long()] >= 0)
+    return pos[s[sel].long()].cpu().numpy(), t[sel].cpu().numpy(), g[sel].cpu().numpy()
+
+
+def test_config4_int8_backbone_full_size(engine):
+    """Config 4 at its stated size (120 000 voxels, int8).  Activation scales are calibrated on this engine's own
+    fp16 pass of config 3 (99.99th percentile, the rule of the reduced-size test).  Checked: the calibrated range is
+    in use on every layer; two eager passes and three graph replays give the same bytes; and on 4 000 sampled output
+    rows of three layers (16->32 strided, 64->64 SubM, 128->128 SubM) the int8 result equals int64 accumulation +
+    the oracle's requantize rule applied to the pairs of the emitted index tensor, bit for bit."""
+    from deploy3d_amd import layers, synth
+    n = 120000
+    cfg3 = synth.config3(n)
+    net3, x3, _ = run_gpu_chain(cfg3)
+    acts = {"input": cfg3["feats"]}
+    acts.update({s["name"]: net3.outputs[s["name"]].feats[:int(net3.outputs[s["name"]].num_act.item())].float().cpu().numpy()
+                 for s in cfg3["layers"]})
+    counts = {s["name"]: int(net3.outputs[s["name"]].num_act.item()) for s in cfg3["layers"] if not s["subm"]}
+    del net3, x3
+    cfg = synth.config4(n, acts)
+    caps = layers.plan_capacities(cfg["layers"], n, counts)
+    net = layers.SparseBackbone(cfg["layers"], cfg["weights"], caps, dtype=torch.int8)
+    x = layers.make_input(cfg["coords"], cfg["feats_q"], cfg["grid"], dtype=torch.int8)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        y = net.forward(x)
+        stream.synchronize()
+        first = {s["name"]: net.outputs[s["name"]].feats.clone() for s in cfg["layers"]}
+        y = net.forward(x)
+        stream.synchronize()
+        for s in cfg["layers"]:
+            assert torch.equal(net.outputs[s["name"]].feats, first[s["name"]]), s["name"]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            y = net.forward(x)
+        for _ in range(3):
+            y.feats.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y.feats, first[cfg["layers"][-1]["name"]])
+    rng = np.random.default_rng(4)
+    prev = "input"
+    for spec, (w, b) in zip(cfg["layers"], cfg["weights"]):
+        out = net.outputs[spec["name"]]
+        n_out = int(out.num_act.item())
+        q = first[spec["name"]][:n_out]
+        assert int(q.abs().max()) >= 100, spec["name"]            # the calibrated range is in use
+        if spec["name"] in ("down1", "conv3_1", "conv4_1"):
+            rb = net.rulebooks[spec["key"]]
+            rows = torch.from_numpy(rng.choice(n_out, size=min(4000, n_out), replace=False)).cuda()
+            xin = x.feats if prev == "input" else first[prev]
+            p, t, g = _sampled_rows_reference(rb, rows, xin, w, None)
+            w_q, s_w = oracle.quantize_weights(w)
+            xi = xin.cpu().numpy().astype(np.int64)
+            acc = np.zeros((len(rows), spec["cout"]), dtype=np.int64)
+            for tap in range(w_q.shape[0]):
+                m_ = t == tap
+                if m_.any():
+                    np.add.at(acc, p[m_], xi[g[m_]] @ w_q[tap].astype(np.int64))
+            assert np.abs(acc).max() < 2 ** 31
+            m, bq = oracle.requant_params(spec["s_in"], s_w, spec["s_out"], b)
+            want = oracle.requantize(acc.astype(np.int32), m, bq, bool(spec.get("relu")))
+            np.testing.assert_array_equal(q[rows].cpu().numpy(), want, err_msg=spec["name"])
+        prev = spec["name"]
+
+
+def test_config5_full_size_first_layers_vs_oracle(engine):
+    """Config 5 at its stated size (250 000 voxels): the two first-level layers of the block (SubM k(3,1,3) and
+    k(1,3,3), 32->64) against the oracle: rulebooks bit-exact in canonical form, features within 2e-2*rms."""
+    from deploy3d_amd import synth
+    cfg = synth.config5()
+    net, x, y = run_gpu_chain(cfg)
+    two = dict(cfg, layers=[s for s in cfg["layers"] if s["name"] in ("a1", "b1")])
+    two["weights"] = [cfg["weights"][cfg["layers"].index(s)] for s in two["layers"]]
+    assert len(two["layers"]) == 2 and {s["key"] for s in two["layers"]} == {"k313", "k133"}
+    ref = chain.oracle_chain(two, threads=8)
+    for spec in two["layers"]:
+        rb = net.rulebooks[spec["key"]]
+        orb = ref["_rulebooks"][spec["key"]]
+        np.testing.assert_array_equal(rb.index.cpu().numpy(), orb["index"], err_msg=spec["key"])
+        out = net.outputs[spec["name"]]
+        got = out.feats[:250000].float().cpu().numpy()
+        want = ref[spec["name"]]["exact"]
+        rms = float(np.sqrt(np.mean(want ** 2)))
+        assert float(np.abs(got - want).max()) <= 2e-2 * rms, spec["name"]

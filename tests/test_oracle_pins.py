@@ -251,3 +251,72 @@ def test_int8_conv_and_requantize_exact():
                              np.array([0.0], np.float32), False)[0, 0] == 127
     assert oracle.requantize(np.array([[-10 ** 9]], np.int32), np.array([1.0], np.float32),
                              np.array([0.0], np.float32), True)[0, 0] == 0
+
+
+def test_quantize_weights_per_output_channel():
+    """oracle.quantize_weights (no counterpart in the reference: it has no int8 path, trt/spconv/mm_trt.cu:184).
+    Pinned by what symmetric per-OUTPUT-channel quantization means, not by its formula: every channel's largest
+    magnitude sits in a different (tap, input channel) and must land on +-127 with a scale that reproduces it; an
+    all-zero channel gets scale 1; every weight is reproduced to within half a quantum.  Taking the maximum over
+    the wrong axes, a per-tensor scale, 128 levels or truncation instead of rounding each fail one of these."""
+    rng = np.random.default_rng(21)
+    kvol, cin, cout = 27, 16, 8
+    w = (rng.standard_normal((kvol, cin, cout)) * 0.01).astype(np.float32)
+    peaks = np.array([0.5, 3.0, 0.125, 7.5, 1.0, 0.75, 2.25, 0.0], dtype=np.float32)
+    where = [(c * 3 % kvol, (5 * c + 1) % cin) for c in range(cout)]
+    for c, (t, ci) in enumerate(where):
+        w[t, ci, c] = peaks[c] * (-1 if c % 2 else 1)
+    w[:, :, 7] = 0.0                                     # a dead channel
+    q, s_w = oracle.quantize_weights(w)
+    assert q.dtype == np.int8 and q.shape == w.shape and s_w.shape == (cout,)
+    for c, (t, ci) in enumerate(where[:7]):
+        assert q[t, ci, c] == (-127 if c % 2 else 127), c
+        assert abs(float(s_w[c]) * 127.0 - float(peaks[c])) <= 1e-12 * float(peaks[c]), c
+        assert np.abs(q[:, :, c]).max() == 127
+    assert s_w[7] == 1.0 and not q[:, :, 7].any()
+    err = np.abs(w.astype(np.float64) - q.astype(np.float64) * s_w[None, None, :])
+    assert (err <= s_w[None, None, :] * (0.5 + 1e-9)).all()
+    assert np.abs(q).max() <= 127 and q.min() >= -127    # symmetric: -128 is never produced
+    # an exact tie between two levels rounds to the even one: 2.5 quanta -> 2, 3.5 quanta -> 4
+    t = np.zeros((1, 4, 1), dtype=np.float32)
+    t[0, :, 0] = [127.0, 2.5, 3.5, -2.5]
+    qt, st = oracle.quantize_weights(t)
+    assert st[0] == 1.0 and qt[0, :, 0].tolist() == [127, 2, 4, -2]
+
+
+def test_requant_params_mean_what_requantization_needs():
+    """oracle.requant_params: with activations x = q_x * s_in, weights w = q_w * s_w[c] and outputs in quanta of
+    s_out, the real pre-activation of an accumulator a is a * s_in * s_w[c] + bias[c], so the output level is
+    rint((a * s_in * s_w[c] + bias[c]) / s_out).  m and bq are checked (1) against exact rational arithmetic,
+    correctly rounded to fp32 up to the double rounding of one division, and (2) end to end through
+    oracle.requantize against that definition evaluated in rationals, away from rounding ties.  A swapped
+    quotient, a missing scale or a bias left in real units fails both."""
+    from fractions import Fraction
+    rng = np.random.default_rng(22)
+    cout = 6
+    s_in, s_out = np.float32(0.0371), np.float32(0.0519)
+    s_w = (rng.random(cout) * 0.01 + 1e-4).astype(np.float64)
+    bias = rng.standard_normal(cout).astype(np.float32)
+    m, bq = oracle.requant_params(s_in, s_w, s_out, bias)
+    assert m.dtype == np.float32 and bq.dtype == np.float32
+    for c in range(cout):
+        m_exact = Fraction(float(s_in)) * Fraction(float(s_w[c])) / Fraction(float(s_out))
+        b_exact = Fraction(float(bias[c])) / Fraction(float(s_out))
+        for got, exact in ((m[c], m_exact), (bq[c], b_exact)):
+            ulp = float(np.spacing(np.float32(abs(float(exact)))))
+            assert abs(Fraction(float(got)) - exact) <= Fraction(ulp) * Fraction(501, 1000), (c, got, float(exact))
+    m0, bq0 = oracle.requant_params(s_in, s_w, s_out, None)
+    assert np.array_equal(m0, m) and not bq0.any()
+    acc = rng.integers(-40000, 40000, (300, cout)).astype(np.int32)
+    for relu in (False, True):
+        q = oracle.requantize(acc, m, bq, relu)
+        for r in range(acc.shape[0]):
+            for c in range(cout):
+                real = (Fraction(int(acc[r, c])) * Fraction(float(s_in)) * Fraction(float(s_w[c])) +
+                        Fraction(float(bias[c]))) / Fraction(float(s_out))
+                frac = real - (real.numerator // real.denominator)
+                if abs(frac - Fraction(1, 2)) < Fraction(1, 100):
+                    continue                                 # fp32 evaluation may fall on the other side of a tie
+                level = int(round(real))
+                level = max(0 if relu else -128, min(127, level))
+                assert q[r, c] == level, (r, c, float(real))
