@@ -18,6 +18,10 @@ constexpr int kSegment = 128;     // tap segments of the index tensor start on m
                                   // (reference: TBSegment, trt/spconv/index.cu:21)
 constexpr int kRbThreads = 256;   // rulebook kernels: 4 wavefronts per workgroup
 
+// Size of the scratch array of d3d_enqueue_static (scratch.hip); D3D_STATIC_SCRATCH_BYTES in the public header.
+constexpr size_t kStaticScratchBytes = static_cast<size_t>(D3D_STATIC_SCRATCH_BYTES);
+int32_t staticScratch(void** ptr, size_t* bytes);
+
 void setError(const char* fmt, ...);
 const char* lastError();
 

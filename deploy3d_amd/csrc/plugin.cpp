@@ -23,6 +23,7 @@ namespace d3d {
 // ---------------------------------------------------------------------------
 namespace {
 thread_local char g_error[512] = "";
+thread_local bool g_noAlloc = false;  // set for the duration of d3d_enqueue_static: no device allocation allowed
 }
 
 void setError(const char* fmt, ...) {
@@ -180,7 +181,7 @@ void noteRulebookWritten(const void* index) {
 // buffer of the entry (null if that fails or D3D_RULEBOOK_NBR=0 asks for the derived form)...
 int32_t* reserveForwardTable(const void* index, int kVol, int64_t outRows) {
   const char* env = std::getenv("D3D_RULEBOOK_NBR");
-  if ((env && env[0] == '0') || outRows <= 0) return nullptr;
+  if ((env && env[0] == '0') || outRows <= 0 || g_noAlloc) return nullptr;
   std::lock_guard<std::mutex> lock(g_cacheMutex);
   NbrTable& t = g_cache[index].forward;
   const size_t bytes = static_cast<size_t>(kVol) * static_cast<size_t>(outRows) * sizeof(int32_t);
@@ -734,6 +735,10 @@ struct MMPlugin final : d3d_plugin {
       setError("SPConvMM: null descriptor or tensor");
       return D3D_ERR_BAD_ARG;
     }
+    if (g_noAlloc) {
+      setError("SPConvMM keeps its neighbour table in library-allocated memory: use d3d_enqueue");
+      return D3D_ERR_UNSUPPORTED;
+    }
     const int32_t dtype = inDesc[0].dtype;
     if (!featureType(dtype) || outDesc[0].dtype != dtype) {
       setError("SPConvMM: feature dtype %d / output dtype %d not implemented", dtype, outDesc[0].dtype);
@@ -1144,6 +1149,22 @@ int32_t d3d_enqueue(d3d_plugin* p, const d3d_tensor_desc* in_desc, const d3d_ten
   D3D_GUARD_BEGIN
   if (!p) return D3D_ERR_BAD_ARG;
   return p->enqueue(in_desc, out_desc, inputs, outputs, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+  D3D_GUARD_END(D3D_ERR_BAD_ARG)
+}
+
+int32_t d3d_enqueue_static(d3d_plugin* p, const d3d_tensor_desc* in_desc, const d3d_tensor_desc* out_desc,
+                           const void* const* inputs, void* const* outputs, void* stream) {
+  D3D_GUARD_BEGIN
+  if (!p) return D3D_ERR_BAD_ARG;
+  void* ws = nullptr;
+  size_t wsBytes = 0;
+  int32_t rc = staticScratch(&ws, &wsBytes);
+  if (rc != D3D_OK) return rc;
+  struct Scope {
+    Scope() { g_noAlloc = true; }
+    ~Scope() { g_noAlloc = false; }
+  } scope;
+  return p->enqueue(in_desc, out_desc, inputs, outputs, ws, wsBytes, static_cast<hipStream_t>(stream));
   D3D_GUARD_END(D3D_ERR_BAD_ARG)
 }
 

@@ -27,7 +27,7 @@ EXPORTS = [
     "d3d_create", "d3d_clone", "d3d_destroy", "d3d_plugin_type", "d3d_plugin_version", "d3d_serialize_size",
     "d3d_serialize", "d3d_num_outputs", "d3d_output_dims", "d3d_output_dtype", "d3d_supports_format",
     "d3d_configure", "d3d_workspace_size", "d3d_enqueue", "d3d_last_error", "d3d_num_ops", "d3d_op_name",
-    "d3d_clear_cache",
+    "d3d_clear_cache", "d3d_enqueue_static",
 ]
 
 
@@ -102,6 +102,8 @@ def load_library(path=None):
     lib.d3d_workspace_size.argtypes = [vp, descp, i32, descp, i32]
     lib.d3d_enqueue.restype = i32
     lib.d3d_enqueue.argtypes = [vp, descp, descp, ctypes.POINTER(vp), ctypes.POINTER(vp), vp, sz, vp]
+    lib.d3d_enqueue_static.restype = i32
+    lib.d3d_enqueue_static.argtypes = [vp, descp, descp, ctypes.POINTER(vp), ctypes.POINTER(vp), vp]
     lib.d3d_last_error.restype = ctypes.c_char_p
     lib.d3d_num_ops.restype = i32
     lib.d3d_op_name.restype = ctypes.c_char_p
@@ -201,12 +203,20 @@ class Plugin:
             for i, t in enumerate(ts):
                 arr[i] = None if t is None or t.numel() == 0 else t.data_ptr()
             return arr
-        ws_ptr = None if workspace is None else workspace.data_ptr()
-        ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+        static = isinstance(workspace, str)
+        ws_ptr = None if workspace is None or static else workspace.data_ptr()
+        ws_bytes = 0 if workspace is None or static else workspace.numel() * workspace.element_size()
         if stream is None:
             stream = torch.cuda.current_stream().cuda_stream
+        if static:  # workspace="static" -> d3d_enqueue_static: the library's own fixed scratch array, no allocation
+            _check(self._lib.d3d_enqueue_static(self._h, _desc_array(in_descs), _desc_array(out_descs), ptrs(inputs),
+                                                ptrs(outputs), ctypes.c_void_p(stream)))
+            return
         _check(self._lib.d3d_enqueue(self._h, _desc_array(in_descs), _desc_array(out_descs), ptrs(inputs),
                                      ptrs(outputs), ws_ptr, ws_bytes, ctypes.c_void_p(stream)))
+
+
+STATIC_SCRATCH_BYTES = 64 << 20
 
 
 def torch_dtype(d3d_dtype):

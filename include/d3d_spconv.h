@@ -138,6 +138,18 @@ int32_t d3d_enqueue(d3d_plugin* p, const d3d_tensor_desc* in_desc, const d3d_ten
                     const void* const* inputs, void* const* outputs, void* workspace, size_t workspace_bytes,
                     void* stream);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory or hand over a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  d3d_enqueue for SPConvIdx{N}d,
+ * BEVDensify and SimpleMeanEncoder with the workspace taken from a fixed array of D3D_STATIC_SCRATCH_BYTES that is
+ * part of the library's device image (each GPU the library runs on holds it until the process ends).  Calls no
+ * hipMalloc / hipFree; an operator whose d3d_workspace_size() exceeds the array returns D3D_ERR_WORKSPACE, and
+ * SPConvMM (which keeps derived tables in library-allocated memory) returns D3D_ERR_UNSUPPORTED.  All calls on one
+ * GPU share the array: calls that overlap in time on one GPU (two streams, two threads) race; calls ordered on
+ * one stream do not, since every operator clears what it needs zeroed itself. */
+#define D3D_STATIC_SCRATCH_BYTES (64u << 20)
+int32_t d3d_enqueue_static(d3d_plugin* p, const d3d_tensor_desc* in_desc, const d3d_tensor_desc* out_desc,
+                           const void* const* inputs, void* const* outputs, void* stream);
+
 /* Text of the last error on the calling thread ("" if none).  Replaces the
  * reference's std::cout reporting (trt/include/common/macros.h:14-34). */
 const char* d3d_last_error(void);
