@@ -526,14 +526,18 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
 // Block-map path.  When the grid is small enough to afford 16 bytes per 64
 // cells, occupancy is kept in a dense table of records instead of the hash:
 //   record = { u64 bits; u32 prefix; u32 pad }   one per block of 64 cells
-// A block is a small brick of the grid (4x4x4 cells in 3-D), so a 3x3x3
-// neighbourhood touches 1-8 records, all close in memory and resident in L2,
-// where a hash probe costs one random cache line per tap.  A voxel's rank is
-// prefix + popcount(bits below its own), i.e. voxels are ranked in brick-major
-// order.  SubM looks rows up through perm[rank]; strided outputs are numbered
-// by their rank directly, which needs no CAS, no owner election, and leaves
-// output rows sorted brick-major, so neighbouring voxels sit in neighbouring
-// feature rows for the convolution's gathers.
+// A block is a small brick of the grid (1x8x8 cells in 3-D: one level of the
+// outermost dim), so a 3x3x3 neighbourhood touches at most 12 records, close
+// in memory and resident in L2, where a hash probe costs one random cache
+// line per tap.  A voxel's rank is prefix + popcount(bits below its own), i.e.
+// voxels are ranked in brick-major order.  SubM looks rows up through
+// perm[rank]; strided outputs are numbered by their rank directly, which
+// needs no CAS, no owner election, and leaves output rows sorted level by
+// level of the outermost dim and in 8x8 patches inside a level.  Rows that
+// follow each other then share most of their neighbourhood pattern (on a
+// LiDAR grid: which of the levels above and below exist), which lets the
+// convolution skip the taps a whole tile of rows lacks, and their neighbours
+// sit in runs of consecutive feature rows for its gathers.
 // ===========================================================================
 struct __attribute__((aligned(16))) BmRecord {
   unsigned long long bits;
@@ -860,18 +864,19 @@ bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* 
 }
 
 // ---------------------------------------------------------------------------
-// "Near" passes of the block-map path.  When, in every dim, the taps of one
-// input reach at most E+1 consecutive output cells (E = brick extent), all
-// targets of that input lie in a 2x2x2 group of bricks.  One thread then
-// serves one input: it fetches that group once (8 independent 16-byte loads,
-// neighbours in memory) and resolves all kVol taps from it, instead of one
-// random record access per (tap, input) pair.  A wavefront's memory requests
+// "Near" passes of the block-map path.  When the taps of one input reach at
+// most 2E+1 consecutive output cells in dim 1 and E+1 in dims 2 and 3 (E =
+// brick extent of the dim), all targets of that input lie in a 3x2x2 group of
+// bricks.  One thread then serves one input: it fetches that group once (12
+// independent 16-byte loads, neighbours in memory) and resolves all kVol taps
+// from it, instead of one random record access per (tap, input) pair.  A wavefront's memory requests
 // drop from 64 lines per tap to a handful per input, which is what bounds
 // these passes: the request rate of scattered accesses, not bandwidth.
 // Requires the outermost of the four dims to be degenerate (always true for
 // 1-D..3-D rulebooks).
 // ---------------------------------------------------------------------------
-constexpr int kNearGroup = 8;
+constexpr int kNearGroup = 12;          // members e = e1 * 4 + e2 * 2 + e3 with e1 in 0..2, e2 and e3 in 0..1
+constexpr int kNearMembers[kMaxSpatial] = {1, 3, 2, 2};
 
 // Lowest output cell (clamped to 0) any tap of input coordinate `in` can reach in `dim`.
 __device__ __forceinline__ int nearBaseCell(const RbGeom& g, int dim, int in) {
@@ -904,9 +909,9 @@ __device__ __forceinline__ NearBase nearBase(const RbGeom& g, const BlockMap& m,
   return b;
 }
 
-// Record index offset and validity of group member e = (e1, e2, e3) in {0,1}^3.
+// Record index offset and validity of group member e = (e1, e2, e3) in {0,1,2} x {0,1}^2.
 __device__ __forceinline__ bool nearMember(const BlockMap& m, const NearBase& b, int e, uint32_t* rec) {
-  const int e1 = (e >> 2) & 1, e2 = (e >> 1) & 1, e3 = e & 1;
+  const int e1 = e >> 2, e2 = (e >> 1) & 1, e3 = e & 1;
   *rec = b.rec0 + static_cast<uint32_t>((e1 * m.nb[2] + e2) * m.nb[3] + e3);
   return b.ok && b.brick[0] < m.nb[0] && b.brick[1] + e1 < m.nb[1] && b.brick[2] + e2 < m.nb[2] &&
          b.brick[3] + e3 < m.nb[3];
@@ -922,7 +927,8 @@ __device__ __forceinline__ void nearForEachTap(const RbGeom& g, const BlockMap& 
   for (int i1 = 0; i1 < g.k[1]; ++i1) {
     int o1;
     const bool ok1 = tapDim(g, 1, c[2], i1, o1) && ok0;
-    const int e1 = (o1 >> m.shift[1]) - b.brick[1];
+    int e1 = (o1 >> m.shift[1]) - b.brick[1];
+    e1 = e1 < 0 ? 0 : (e1 > 2 ? 2 : e1);  // in range by construction when the tap is valid
     for (int i2 = 0; i2 < g.k[2]; ++i2) {
       int o2;
       const bool ok2 = tapDim(g, 2, c[3], i2, o2) && ok1;
@@ -935,7 +941,7 @@ __device__ __forceinline__ void nearForEachTap(const RbGeom& g, const BlockMap& 
         bit = (bit << m.shift[1]) | (static_cast<uint32_t>(o1) & ((1u << m.shift[1]) - 1));
         bit = (bit << m.shift[2]) | (static_cast<uint32_t>(o2) & ((1u << m.shift[2]) - 1));
         bit = (bit << m.shift[3]) | (static_cast<uint32_t>(o3) & ((1u << m.shift[3]) - 1));
-        f(tap, ok3, ((e1 & 1) << 2) | ((e2 & 1) << 1) | (e3 & 1), bit);
+        f(tap, ok3, (e1 << 2) | ((e2 & 1) << 1) | (e3 & 1), bit);
         ++tap;
       }
     }
@@ -964,7 +970,8 @@ __device__ __forceinline__ void nearForEachTapFixed(const RbGeom& g, const Block
         const int num = c[dim + 1] + g.p[dim] - i;
         const int o = num >> ls;
         ok[q][i] = num >= 0 && (num & (st - 1)) == 0 && o < g.shape[dim + 1];
-        member[q][i] = ((o >> m.shift[dim]) - b.brick[dim]) & 1;
+        const int mem = (o >> m.shift[dim]) - b.brick[dim];
+        member[q][i] = q == 0 ? (mem < 0 ? 0 : (mem > 2 ? 2 : mem)) : (mem & 1);
         part[q][i] = static_cast<uint32_t>(o) & ((1u << m.shift[dim]) - 1);
       } else {
         ok[q][i] = false;
@@ -996,7 +1003,7 @@ __device__ __forceinline__ void nearTaps(const RbGeom& g, const BlockMap& m, con
   else nearForEachTap(g, m, c, b, f);
 }
 
-// Record indices of the 8 group members; members outside the grid are clamped to record 0 (so that every
+// Record indices of the group members; members outside the grid are clamped to record 0 (so that every
 // load is unconditional and all eight issue back to back) and reported absent in the returned mask.
 __device__ __forceinline__ uint32_t nearMembers(const BlockMap& m, const NearBase& b, uint32_t rec[kNearGroup]) {
   uint32_t present = 0;
@@ -1164,7 +1171,7 @@ namespace {
 // Brick shape per number of real spatial dims (extents multiply to 64).
 BlockMap makeBlockMap(const RbGeom& g, uint64_t* records) {
   static const int kShifts[kMaxSpatial + 1][kMaxSpatial] = {
-      {0, 0, 0, 6}, {0, 0, 0, 6}, {0, 0, 3, 3}, {0, 2, 2, 2}, {1, 1, 2, 2}};
+      {0, 0, 0, 6}, {0, 0, 0, 6}, {0, 0, 3, 3}, {0, 0, 3, 3}, {1, 1, 2, 2}};
   BlockMap m{};
   uint64_t n = static_cast<uint64_t>(g.shape[0] > 0 ? g.shape[0] : 0);
   for (int dim = 0; dim < kMaxSpatial; ++dim) {
@@ -1243,12 +1250,12 @@ RbWorkspace planWith(const RbGeom& g, int64_t cap, bool subM, bool blockMap) {
   return w;
 }
 
-// True if every input's targets fall in one 2x2x2 group of bricks (see the "near" passes).
+// True if every input's targets fall in one 3x2x2 group of bricks (see the "near" passes).
 bool nearEligible(const RbGeom& g, const BlockMap& m) {
   if (g.k[0] != 1) return false;
   for (int dim = 1; dim < kMaxSpatial; ++dim) {
     const int reach = g.transpose ? (g.k[dim] - 1) * g.d[dim] : ((g.k[dim] - 1) * g.d[dim]) / g.s[dim];
-    if (reach > (1 << m.shift[dim])) return false;
+    if (reach > ((kNearMembers[dim] - 1) << m.shift[dim])) return false;
   }
   const char* e = std::getenv("D3D_RULEBOOK_NEAR");
   return !(e && e[0] == '0');
