@@ -20,9 +20,16 @@ OBJ = os.path.join(LIBS, "obj")
 ENGINE_LIB = os.path.join(LIBS, "libdeploy3d_amd.so")
 SYNTH_LIB = os.path.join(LIBS, "libd3d_synth.so")
 
-ENGINE_SOURCES = ["rulebook.hip", "conv.hip", "conv_half.hip", "conv_bf16.hip", "conv_int8.hip", "densify.hip",
-                  "voxelize.hip", "scratch.hip", "plugin.cpp"]
-ENGINE_HEADERS = ["common.h", "conv_kernels.h", os.path.join(ROOT, "include", "d3d_spconv.h")]
+ENGINE_SOURCES = ["rulebook.hip", "conv.hip", "conv_half.hip", "conv_bf16.hip", "conv_int8.hip", "conv_pipe_half.hip",
+                  "conv_pipe_bf16.hip", "densify.hip", "voxelize.hip", "scratch.hip", "plugin.cpp"]
+ENGINE_HEADERS = ["common.h", "conv_kernels.h", "conv_pipe.h", os.path.join(ROOT, "include", "d3d_spconv.h")]
+# per-source extra flags
+EXTRA_FLAGS = {
+    # keeps the MFMA accumulators of the pipelined kernel in VGPRs (see the header of the two files)
+    "conv_pipe_half.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "conv_pipe_bf16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+PEAKS_BIN = os.path.join(LIBS, "d3d_peaks")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
@@ -68,7 +75,7 @@ def build_engine(verbose=False, incremental=False, jobs=None):
     for src in _existing_sources():
         obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
         objs.append(obj)
-        stamp = _stamp(src, flags)
+        stamp = _stamp(src, flags + EXTRA_FLAGS.get(src, []))
         stamp_file = obj + ".stamp"
         fresh = False
         if incremental and os.path.exists(obj) and os.path.exists(stamp_file):
@@ -79,7 +86,7 @@ def build_engine(verbose=False, incremental=False, jobs=None):
 
     def compile_one(item):
         src, obj, stamp = item
-        out = _run([_hipcc()] + flags + ["-c", os.path.join(CSRC, src), "-o", obj])
+        out = _run([_hipcc()] + flags + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj])
         with open(obj + ".stamp", "w") as f:
             f.write(stamp)
         return src, out
@@ -95,6 +102,13 @@ def build_engine(verbose=False, incremental=False, jobs=None):
     return ENGINE_LIB
 
 
+def build_peaks():
+    """The measured-peaks microbenchmark (dense MFMA loop, streaming copy), a standalone program bench.py runs."""
+    os.makedirs(LIBS, exist_ok=True)
+    _run([_hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17", os.path.join(CSRC, "peaks.hip"), "-o", PEAKS_BIN])
+    return PEAKS_BIN
+
+
 def build_synth():
     os.makedirs(LIBS, exist_ok=True)
     cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
@@ -106,6 +120,9 @@ def build_synth():
 def build_all(verbose=False, incremental=False):
     build_synth()
     build_engine(verbose=verbose, incremental=incremental)
+    if not (incremental and os.path.exists(PEAKS_BIN) and
+            os.path.getmtime(PEAKS_BIN) >= os.path.getmtime(os.path.join(CSRC, "peaks.hip"))):
+        build_peaks()
 
 
 if __name__ == "__main__":

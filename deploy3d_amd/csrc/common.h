@@ -85,6 +85,10 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
 int32_t launchBuildNeighbours(const int32_t* index, int64_t rowLen, const int32_t* numIndex, bool inverse, int kVol,
                               int64_t outRows, int32_t* nbr, hipStream_t stream);
 
+// masks[i] = taps (bit t) that any of output rows 64i..64i+63 has, from a neighbour table; kVol <= 64
+int32_t launchTileMasks(const int32_t* nbr, int64_t pitch, int tapMirror, int kVol, int64_t outRows, int64_t inRows,
+                        unsigned long long* masks, hipStream_t stream);
+
 struct ConvArgs {
   int32_t dtype;          // D3D_FLOAT / D3D_HALF / D3D_BF16 / D3D_INT8
   int kVol, cin, cout;
@@ -97,14 +101,27 @@ struct ConvArgs {
   const float* bias;      // device fp32 [cout] or null
   const float* requantM;  // int8: per-channel multiplier
   const float* requantB;  // int8: per-channel bias in output quanta
-  const int32_t* nbr;     // [kVol, outRows]
+  const int32_t* nbr;     // [kVol, nbrPitch]: input row that feeds output row r through tap t, at nbr[t' * nbrPitch + r]
+                          // with t' = tapMirror ? kVol - 1 - t : t; -1 (or any value >= inRows) = no neighbour
+  int64_t nbrPitch;       // row pitch of nbr in elements; 0 = outRows
+  int tapMirror;          // the table is indexed by the mirrored tap (a SubM rulebook's input-major table, see rbCompact)
+  const unsigned long long* tileMasks;  // optional [ceil(outRows / 64)]: bit t set iff any of rows 64i..64i+63 has tap t
   const void* zeros;      // device, >= 512 zero bytes: the row that absent neighbours gather
   int relu;
   int tileRows;           // 0 = choose; else rows per workgroup of the weight-streaming MFMA kernel (128, 256, 512)
   int staged;             // staged MFMA kernel: 0 = choose, -1 = do not use it, else MT | WAVES << 8 | NS << 16 | resident << 24
+  int pipe;               // software-pipelined kernel: 0 = use it where it applies, -1 = do not
 };
 
 int32_t launchConv(const ConvArgs& a, hipStream_t stream);
+// The MFMA kernel family, one translation unit per storage type (conv_half.hip, conv_bf16.hip, conv_int8.hip);
+// D3D_ERR_UNSUPPORTED when no instantiation fits the layer.
+int32_t launchMfmaHalf(const ConvArgs& a, hipStream_t stream);
+int32_t launchMfmaBf16(const ConvArgs& a, hipStream_t stream);
+int32_t launchMfmaInt8(const ConvArgs& a, hipStream_t stream);
+// The software-pipelined kernel (conv_pipe.h): 32 / 64 / 128 channels, kernel volumes up to 64.
+int32_t launchPipeHalf(const ConvArgs& a, hipStream_t stream);
+int32_t launchPipeBf16(const ConvArgs& a, hipStream_t stream);
 
 // True if the MFMA kernel family covers (dtype, cin, cout); otherwise the
 // narrow-channel kernel runs.

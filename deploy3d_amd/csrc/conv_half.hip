@@ -1,0 +1,8 @@
+// Instantiates the MFMA convolution kernels (conv_kernels.h) for one storage type.
+#include "conv_kernels.h"
+
+namespace d3d {
+
+int32_t launchMfmaHalf(const ConvArgs& a, hipStream_t stream) { return convk::launchMfma<_Float16>(a, stream); }
+
+}  // namespace d3d

@@ -788,6 +788,15 @@ struct MMPlugin final : d3d_plugin {
     a.nbr = static_cast<const int32_t*>(table->ptr);
     a.relu = relu ? 1 : 0;
     a.zeros = zeros;
+    if (std::getenv("D3D_TMP_MASKS") && kernelVol <= 64) {  // experiment: masks from a kernel of their own
+      static DeviceBuffer tmpMasks;
+      rc = tmpMasks.reserve(static_cast<size_t>((outRows + 63) / 64 + 1) * 8);
+      if (rc != D3D_OK) return rc;
+      rc = launchTileMasks(a.nbr, outRows, 0, kernelVol, outRows, a.inRows, static_cast<unsigned long long*>(tmpMasks.ptr), stream);
+      if (rc != D3D_OK) return rc;
+      a.tileMasks = static_cast<const unsigned long long*>(tmpMasks.ptr);
+    }
+    if (const char* e = std::getenv("D3D_CONV_PIPE")) a.pipe = e[0] == '0' ? -1 : 0;
     a.tileRows = tileRowsOverride();
     a.staged = stagedOverride();
     return launchConv(a, stream);
