@@ -8,6 +8,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 
 #include "d3d_spconv.h"
 
@@ -21,6 +22,13 @@ constexpr int kRbThreads = 256;   // rulebook kernels: 4 wavefronts per workgrou
 // Size of the scratch array of d3d_enqueue_static (scratch.hip); D3D_STATIC_SCRATCH_BYTES in the public header.
 constexpr size_t kStaticScratchBytes = static_cast<size_t>(D3D_STATIC_SCRATCH_BYTES);
 int32_t staticScratch(void** ptr, size_t* bytes);
+
+// Tuning and test switches (D3D_RULEBOOK, D3D_CONV_STAGED, ...) are honoured only in a process that had
+// D3D_DEBUG_ENV set when the library first looked; otherwise a query costs one cached flag, not a getenv.
+inline const char* debugEnv(const char* name) {
+  static const bool enabled = std::getenv("D3D_DEBUG_ENV") != nullptr;
+  return enabled ? std::getenv(name) : nullptr;
+}
 
 void setError(const char* fmt, ...);
 const char* lastError();
@@ -71,23 +79,35 @@ RbWorkspace planRulebookWorkspace(const RbGeom& g, int64_t cap, bool subM, size_
 // Workspace that is enough for whichever structure gets chosen.  gridKnown = g.shape holds the real output grid.
 size_t rulebookWorkspaceBytes(const RbGeom& g, int64_t cap, bool subM, bool gridKnown);
 
+// By-products of a rulebook build for the convolutions that follow it, and the state that lets a pass reuse the
+// index tensor of the pass before it.  All pointers are device memory owned by the caller of launchRulebook.
+struct RbSide {
+  int32_t* nbr = nullptr;               // [kVol, nbrRows] pairs in output-major form: nbr[tap][output row] = input
+                                        // row, -1 elsewhere; 16-byte aligned; null = not wanted
+  int64_t nbrRows = 0;
+  unsigned long long* masks = nullptr;  // [nMasks] bit t of masks[r / 64]: some output row of 64r..64r+63 has tap t;
+                                        // written with the table of a SubM rulebook when kVol <= 64 (entries past
+                                        // the rows read 0), see masksWritten
+  int64_t nMasks = 0;
+  uint32_t* fillState = nullptr;        // 2 words: end of the used part of the index tensor after the previous
+                                        // pass / after this pass
+  bool incrementalFill = false;         // the index tensor still holds the previous pass that used this fillState:
+                                        // only the slots that pass used and this one does not are set to -1
+  bool masksWritten = false;            // out: this build wrote `masks` (SubM rulebooks with a mirrored table)
+};
+
 // Builds one rulebook on `stream`.  coors [cap, nd+1]; numActIn device int32.
 // index [3, rowLen] with rowLen = kVol * (cap + 128).  outCoors / numActOut are
-// null for SubM.  When nbrOut is given (16-byte aligned, [kVol, nbrRows]) the pairs are also written in
-// output-major form, nbrOut[tap][output row] = input row, -1 elsewhere.  Returns a D3D status.
+// null for SubM.  Returns a D3D status.
 int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const int32_t* numActIn, int64_t cap,
                        int32_t maxNumActOut, int32_t* index, int32_t* numIndex, int32_t* outCoors, int32_t* numActOut,
-                       void* workspace, size_t workspaceBytes, int32_t* nbrOut, int64_t nbrRows, hipStream_t stream);
+                       void* workspace, size_t workspaceBytes, RbSide& side, hipStream_t stream);
 
 // Out-major neighbour table of one rulebook: nbr[tap, row] = gathered input row
 // or -1, rows = maxNumActOut.  Built from the index tensor (optionally with the
 // gather and scatter rows swapped for an inverse convolution).
 int32_t launchBuildNeighbours(const int32_t* index, int64_t rowLen, const int32_t* numIndex, bool inverse, int kVol,
                               int64_t outRows, int32_t* nbr, hipStream_t stream);
-
-// masks[i] = taps (bit t) that any of output rows 64i..64i+63 has, from a neighbour table; kVol <= 64
-int32_t launchTileMasks(const int32_t* nbr, int64_t pitch, int tapMirror, int kVol, int64_t outRows, int64_t inRows,
-                        unsigned long long* masks, hipStream_t stream);
 
 struct ConvArgs {
   int32_t dtype;          // D3D_FLOAT / D3D_HALF / D3D_BF16 / D3D_INT8
@@ -100,7 +120,6 @@ struct ConvArgs {
   const void* weightsMfma;  // device storage-type, MFMA fragment-major (see MMPlugin::configure) or null
   const float* bias;      // device fp32 [cout] or null
   const float* requantM;  // int8: per-channel multiplier
-  const float* requantB;  // int8: per-channel bias in output quanta
   const int32_t* nbr;     // [kVol, nbrPitch]: input row that feeds output row r through tap t, at nbr[t' * nbrPitch + r]
                           // with t' = tapMirror ? kVol - 1 - t : t; -1 (or any value >= inRows) = no neighbour
   int64_t nbrPitch;       // row pitch of nbr in elements; 0 = outRows

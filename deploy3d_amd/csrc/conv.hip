@@ -48,33 +48,10 @@ nbrScatter(const int32_t* __restrict__ gather, const int32_t* __restrict__ scatt
     if (t < 0 || t >= kVol) continue;  // padding slot
     const int32_t o = scatter[j];
     if (o < 0 || o >= outRows) continue;
-    nbr[static_cast<int64_t>(t) * outRows + o] = gather[j];
+    // An index tensor that names two inputs for one (tap, output) - duplicate coordinates, a tensor of other
+    // origin - keeps the higher input row: one neighbour per (tap, output), the same one on every run.
+    atomicMax(&nbr[static_cast<int64_t>(t) * outRows + o], gather[j]);
   }
-}
-
-// masks[i] bit t = some row of 64i..64i+63 has tap t (kVol <= 64); one wavefront per 64 rows
-__global__ void __launch_bounds__(256)
-nbrTileMasks(const int32_t* __restrict__ nbr, int64_t pitch, int tapMirror, int kVol, int64_t outRows, int64_t inRows,
-             unsigned long long* __restrict__ masks) {
-  const int64_t tile = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (tile * 64 >= outRows) return;
-  int64_t row = tile * 64 + lane;
-  if (row >= outRows) row = outRows - 1;
-  const uint32_t limit = static_cast<uint32_t>(inRows);
-  unsigned long long m = 0;
-  for (int t0 = 0; t0 < kVol; t0 += 16) {
-    uint32_t v[16];
-#pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      const int t = t0 + q < kVol ? t0 + q : kVol - 1;
-      v[q] = static_cast<uint32_t>(nbr[static_cast<int64_t>(tapMirror ? kVol - 1 - t : t) * pitch + row]);
-    }
-#pragma unroll
-    for (int q = 0; q < 16; ++q)
-      if (t0 + q < kVol && __ballot(v[q] < limit) != 0ull) m |= 1ull << (t0 + q);
-  }
-  if (lane == 0) masks[tile] = m;
 }
 
 // ---------------------------------------------------------------------------
@@ -262,16 +239,6 @@ int32_t launchBuildNeighbours(const int32_t* index, int64_t rowLen, const int32_
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(nbrScatter, dim3(blocks), dim3(256), 0, stream, gather, scatter, index + 2 * rowLen, numIndex,
                      rowLen, kVol, outRows, nbr);
-  D3D_HIP_CHECK(hipGetLastError());
-  return D3D_OK;
-}
-
-int32_t launchTileMasks(const int32_t* nbr, int64_t pitch, int tapMirror, int kVol, int64_t outRows, int64_t inRows,
-                        unsigned long long* masks, hipStream_t stream) {
-  if (outRows <= 0 || kVol > 64) return D3D_OK;
-  const int64_t tiles = (outRows + 63) / 64;
-  hipLaunchKernelGGL(nbrTileMasks, dim3(static_cast<unsigned>((tiles + 3) / 4)), dim3(256), 0, stream, nbr, pitch,
-                     tapMirror, kVol, outRows, inRows, masks);
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;
 }

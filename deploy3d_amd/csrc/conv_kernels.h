@@ -4,6 +4,8 @@
 #pragma once
 #include <hip/hip_fp16.h>
 
+#include <atomic>
+
 #include "common.h"
 
 namespace d3d {
@@ -830,11 +832,13 @@ constexpr size_t mfmaLds(int kVol, int rows, size_t elem) {
 }
 
 template <class K>
-int32_t grantLds(K kernel, size_t lds, size_t* granted) {
-  if (lds > *granted) {  // dynamic LDS beyond 64 KiB has to be requested per kernel
+int32_t grantLds(K kernel, size_t lds, std::atomic<size_t>* granted) {
+  // dynamic LDS beyond 64 KiB has to be requested per kernel; two threads that both find it not yet granted both
+  // request it, which is harmless
+  if (lds > granted->load(std::memory_order_acquire)) {
     D3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(kLdsLimit)));
-    *granted = kLdsLimit;
+    granted->store(kLdsLimit, std::memory_order_release);
   }
   return D3D_OK;
 }
@@ -847,7 +851,7 @@ int32_t launchMfmaTile(const ConvArgs& a, hipStream_t stream) {
     setError("conv: kernel volume %d too large for the MFMA kernel", a.kVol);
     return D3D_ERR_UNSUPPORTED;
   }
-  static size_t granted = 64 * 1024;
+  static std::atomic<size_t> granted{64 * 1024};
   const int32_t rc = grantLds(&convMfma<T, CIN, COUT, MT, WAVES>, lds, &granted);
   if (rc != D3D_OK) return rc;
   const int tiles = static_cast<int>((a.outRows + TM - 1) / TM);
@@ -863,7 +867,7 @@ template <class T, int CIN, int COUT>
 int32_t launchMfmaResident(const ConvArgs& a, hipStream_t stream) {
   constexpr int WAVES = 16;
   const size_t lds = static_cast<size_t>(a.kVol) * CIN * COUT * sizeof(T) + static_cast<size_t>(WAVES) * a.kVol * 16 * 4;
-  static size_t granted = 64 * 1024;
+  static std::atomic<size_t> granted{64 * 1024};
   const int32_t rc = grantLds(&convMfmaResident<T, CIN, COUT, WAVES>, lds, &granted);
   if (rc != D3D_OK) return rc;
   const int groups = static_cast<int>((a.outRows + 15) / 16);
@@ -891,7 +895,7 @@ int32_t launchStagedCfg(const ConvArgs& a, hipStream_t stream) {
                      static_cast<size_t>(WAVES) * NS * WM * CH * 16;
   if (lds > kLdsLimit) return D3D_ERR_UNSUPPORTED;  // the caller falls back
   if (static_cast<uint64_t>(a.inRows) * CIN * sizeof(T) >= (1ull << 32)) return D3D_ERR_UNSUPPORTED;  // 32-bit row offsets
-  static size_t granted = 64 * 1024;
+  static std::atomic<size_t> granted{64 * 1024};
   const int32_t rc = grantLds(&convStaged<T, CIN, COUT, KS, MT, WAVES, NS, RESIDENT>, lds, &granted);
   if (rc != D3D_OK) return rc;
   const int tiles = static_cast<int>((a.outRows + TM - 1) / TM);

@@ -387,7 +387,7 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
       static_cast<uint64_t>(a.kVol) * static_cast<uint64_t>(pitch) * 4 >= 0xFFFF0000ull ||
       static_cast<uint64_t>(a.outRows) + TM >= 0x3FFFFFFFull)
     return D3D_ERR_UNSUPPORTED;                         // 32-bit buffer offsets
-  static size_t granted = 64 * 1024;
+  static std::atomic<size_t> granted{64 * 1024};
   const int32_t rc = grantLds(&convPipe<T, CIN, COUT, MT, WAVES, DBG>, lds, &granted);
   if (rc != D3D_OK) return rc;
   const int tiles = static_cast<int>((a.outRows + TM - 1) / TM);

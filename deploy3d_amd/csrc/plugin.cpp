@@ -147,94 +147,31 @@ int dtypeBytes(int32_t dtype) {
 }
 
 // ---------------------------------------------------------------------------
-// neighbour-table cache: one entry per index tensor (the value an indice key
-// names in the calling graph).  The rulebook operator bumps the generation of
-// its output tensor; the first convolution that consumes a generation builds
-// the table, the other convolutions sharing the key reuse it.  An index
-// tensor this library did not produce has no generation to trust, so its
-// table is rebuilt on every convolution.
+// Rulebook by-products.  A rulebook operator that convolutions have been linked to (d3d_link_rulebook) writes,
+// besides the index tensor, the pairs in output-major form (the neighbour table the convolution kernels read) and
+// the tap masks of 64-row tiles, into device memory this record owns.  The record belongs to the operator handle
+// and to the convolutions linked to it (shared ownership: it is freed when the last of them is destroyed), and a
+// convolution uses it only for the index tensor the operator wrote last, at the shapes it wrote it for; any other
+// index tensor has its table derived from its contents on every enqueue, as the reference re-reads the index on
+// every enqueue (trt/spconv/mm_trt.cu:166-170).
 // ---------------------------------------------------------------------------
-struct NbrTable {
-  std::shared_ptr<DeviceBuffer> buf;
-  uint64_t builtGeneration = 0;
-  bool built = false;
+struct RulebookLink {
+  std::mutex mutex;
+  bool wanted = false;            // some convolution is linked: the operator writes the table
+  bool wantMasks = false;         // ... and one of them runs a kernel that reads tile masks
+  DeviceBuffer table, masks, fillState;
+  // what the table describes (set by the operator's enqueue)
+  const void* index = nullptr;    // index tensor the by-products belong to
+  const void* numIndex = nullptr;
   int kVol = 0;
   int64_t outRows = 0, rowLen = 0;
-  const void* numIndex = nullptr;
+  bool tableValid = false, masksValid = false;
+  // incremental fill: index tensor that holds a complete earlier pass of this operator
+  const void* primedIndex = nullptr;
+  int64_t primedRowLen = 0;
 };
-struct NbrEntry {
-  bool managed = false;
-  uint64_t generation = 0;
-  NbrTable forward, inverse;
-};
-std::mutex g_cacheMutex;
-std::unordered_map<const void*, NbrEntry> g_cache;
 
-void noteRulebookWritten(const void* index) {
-  std::lock_guard<std::mutex> lock(g_cacheMutex);
-  NbrEntry& e = g_cache[index];
-  e.managed = true;
-  ++e.generation;
-}
-
-// The rulebook operator can write the forward table itself while it compacts the pairs.  This reserves the
-// buffer of the entry (null if that fails or D3D_RULEBOOK_NBR=0 asks for the derived form)...
-int32_t* reserveForwardTable(const void* index, int kVol, int64_t outRows) {
-  const char* env = std::getenv("D3D_RULEBOOK_NBR");
-  if ((env && env[0] == '0') || outRows <= 0 || g_noAlloc) return nullptr;
-  std::lock_guard<std::mutex> lock(g_cacheMutex);
-  NbrTable& t = g_cache[index].forward;
-  const size_t bytes = static_cast<size_t>(kVol) * static_cast<size_t>(outRows) * sizeof(int32_t);
-  if (!t.buf || t.buf->bytes < bytes) {
-    auto nb = std::make_shared<DeviceBuffer>();
-    if (nb->reserve(bytes) != D3D_OK) return nullptr;
-    t.buf = nb;
-    t.built = false;
-  }
-  return static_cast<int32_t*>(t.buf->ptr);
-}
-
-// ... and this records, with the new generation, that the table in it is current.
-void noteForwardTableWritten(const void* index, int kVol, int64_t outRows, int64_t rowLen, const void* numIndex) {
-  std::lock_guard<std::mutex> lock(g_cacheMutex);
-  NbrEntry& e = g_cache[index];
-  NbrTable& t = e.forward;
-  t.built = true;
-  t.builtGeneration = e.generation;
-  t.kVol = kVol;
-  t.outRows = outRows;
-  t.rowLen = rowLen;
-  t.numIndex = numIndex;
-}
-
-int32_t neighbourTable(const int32_t* index, int64_t rowLen, const int32_t* numIndex, bool inverse, int kVol,
-                       int64_t outRows, hipStream_t stream, std::shared_ptr<DeviceBuffer>* out) {
-  std::lock_guard<std::mutex> lock(g_cacheMutex);
-  NbrEntry& e = g_cache[index];
-  NbrTable& t = inverse ? e.inverse : e.forward;
-  const bool fresh = e.managed && t.built && t.builtGeneration == e.generation && t.kVol == kVol &&
-                     t.outRows == outRows && t.rowLen == rowLen && t.numIndex == numIndex;
-  if (!fresh) {
-    const size_t bytes = static_cast<size_t>(kVol) * static_cast<size_t>(outRows) * sizeof(int32_t);
-    if (!t.buf || t.buf->bytes < bytes) {
-      auto nb = std::make_shared<DeviceBuffer>();
-      int32_t rc = nb->reserve(bytes > 0 ? bytes : 4);
-      if (rc != D3D_OK) return rc;
-      t.buf = nb;  // an older table stays alive while an enqueued kernel's owner still holds it
-    }
-    int32_t rc = launchBuildNeighbours(index, rowLen, numIndex, inverse, kVol, outRows,
-                                       static_cast<int32_t*>(t.buf->ptr), stream);
-    if (rc != D3D_OK) return rc;
-    t.built = true;
-    t.builtGeneration = e.generation;
-    t.kVol = kVol;
-    t.outRows = outRows;
-    t.rowLen = rowLen;
-    t.numIndex = numIndex;
-  }
-  *out = t.buf;
-  return D3D_OK;
-}
+size_t maskEntries(int64_t outRows) { return static_cast<size_t>((outRows + 63) / 64 + 8); }
 
 // ---------------------------------------------------------------------------
 // packed little-endian blob reader
@@ -276,6 +213,10 @@ struct d3d_plugin {
   virtual size_t workspaceSize(const d3d_tensor_desc* in, int32_t nbIn) const = 0;
   virtual int32_t enqueue(const d3d_tensor_desc* inDesc, const d3d_tensor_desc* outDesc, const void* const* inputs,
                           void* const* outputs, void* workspace, size_t workspaceBytes, hipStream_t stream) = 0;
+  virtual int32_t setOption(int32_t option, int64_t) {
+    d3d::setError("%s: option %d not known to this operator", type.c_str(), option);
+    return D3D_ERR_UNSUPPORTED;
+  }
 };
 
 namespace d3d {
@@ -289,6 +230,8 @@ struct IdxPlugin final : d3d_plugin {
       outPadding[kMaxSpatial];
   int32_t maxNumActOut = 0;
   bool subM = false, transpose = false;
+  bool persistentIndex = false;                  // D3D_OPT_PERSISTENT_INDEX
+  std::shared_ptr<RulebookLink> link = std::make_shared<RulebookLink>();  // by-products for linked convolutions
 
   int kVol() const {
     int v = 1;
@@ -330,8 +273,39 @@ struct IdxPlugin final : d3d_plugin {
     return D3D_OK;
   }
 
-  d3d_plugin* clone() const override { return new IdxPlugin(*this); }
+  d3d_plugin* clone() const override {
+    auto* c = new IdxPlugin(*this);
+    c->link = std::make_shared<RulebookLink>();  // a clone is another node: its own by-products, no links yet
+    c->persistentIndex = false;
+    return c;
+  }
   int32_t numOutputs() const override { return subM ? 2 : 5; }  // index_trt.cu:98-101
+
+  // Called when a convolution is linked: from now on enqueue also writes the neighbour table and the tile masks.
+  int32_t wantByProducts(bool masks) {
+    std::lock_guard<std::mutex> lock(link->mutex);
+    link->wantMasks = link->wantMasks || (masks && kVol() <= 64);
+    if (maxNumActOut > 0) {
+      int32_t rc = link->table.reserve(static_cast<size_t>(kVol()) * static_cast<size_t>(maxNumActOut) * sizeof(int32_t));
+      if (rc != D3D_OK) return rc;
+      rc = link->masks.reserve(maskEntries(maxNumActOut) * sizeof(unsigned long long));
+      if (rc != D3D_OK) return rc;
+    }
+    link->wanted = true;
+    return D3D_OK;
+  }
+
+  int32_t setOption(int32_t option, int64_t value) override {
+    if (option != D3D_OPT_PERSISTENT_INDEX) return d3d_plugin::setOption(option, value);
+    std::lock_guard<std::mutex> lock(link->mutex);
+    if (value) {
+      int32_t rc = link->fillState.reserve(256);
+      if (rc != D3D_OK) return rc;
+    }
+    persistentIndex = value != 0;
+    link->primedIndex = nullptr;
+    return D3D_OK;
+  }
 
   // spatial extents of the output grid from those of the input grid
   void outSpatial(const int32_t* in, int32_t* out) const {
@@ -450,16 +424,43 @@ struct IdxPlugin final : d3d_plugin {
       }
     }
     const RbGeom g = geometry(grid);
-    int32_t* nbr = reserveForwardTable(outputs[0], kVol(), maxNumActOut);
+    std::lock_guard<std::mutex> lock(link->mutex);
+    RbSide side{};
+    const size_t tableBytes = static_cast<size_t>(kVol()) * static_cast<size_t>(maxNumActOut) * sizeof(int32_t);
+    const bool withTable = link->wanted && maxNumActOut > 0 && link->table.bytes >= tableBytes &&
+                           link->masks.bytes >= maskEntries(maxNumActOut) * sizeof(unsigned long long);
+    if (withTable) {
+      side.nbr = static_cast<int32_t*>(link->table.ptr);
+      side.nbrRows = maxNumActOut;
+      if (link->wantMasks) {
+        side.masks = static_cast<unsigned long long*>(link->masks.ptr);
+        side.nMasks = static_cast<int64_t>(maskEntries(maxNumActOut));
+      }
+    }
+    if (persistentIndex && link->fillState.ptr) {
+      side.fillState = static_cast<uint32_t*>(link->fillState.ptr);
+      side.incrementalFill = link->primedIndex == outputs[0] && link->primedRowLen == rowLen;
+    }
+    link->tableValid = link->masksValid = false;
+    link->primedIndex = nullptr;
     int32_t rc = launchRulebook(g, subM, static_cast<const int32_t*>(inputs[0]),
                                 static_cast<const int32_t*>(inputs[1]), cap, maxNumActOut,
                                 static_cast<int32_t*>(outputs[0]), static_cast<int32_t*>(outputs[1]),
                                 subM ? nullptr : static_cast<int32_t*>(outputs[2]),
-                                subM ? nullptr : static_cast<int32_t*>(outputs[3]), workspace, workspaceBytes, nbr,
-                                maxNumActOut, stream);
+                                subM ? nullptr : static_cast<int32_t*>(outputs[3]), workspace, workspaceBytes, side,
+                                stream);
     if (rc == D3D_OK) {
-      noteRulebookWritten(outputs[0]);
-      if (nbr) noteForwardTableWritten(outputs[0], kVol(), maxNumActOut, rowLen, outputs[1]);
+      link->index = outputs[0];
+      link->numIndex = outputs[1];
+      link->kVol = kVol();
+      link->outRows = maxNumActOut;
+      link->rowLen = rowLen;
+      link->tableValid = withTable;
+      link->masksValid = withTable && side.masksWritten;
+      if (side.fillState) {
+        link->primedIndex = outputs[0];
+        link->primedRowLen = rowLen;
+      }
     }
     return rc;
   }
@@ -484,18 +485,18 @@ const void* zeroRow() {
 // Tuning / test hook: D3D_CONV_TILE_ROWS = rows per workgroup of the weight-streaming MFMA convolution
 // (64 .. 512, a multiple of 64), D3D_CONV_WAVES = 4 or 8 wavefronts per workgroup; unset = heuristic.
 int tileRowsOverride() {
-  const char* e = std::getenv("D3D_CONV_TILE_ROWS");
+  const char* e = debugEnv("D3D_CONV_TILE_ROWS");
   if (!e) return 0;
   const int v = std::atoi(e);
   if (v < 64 || v > 512 || v % 64) return 0;
-  const char* w = std::getenv("D3D_CONV_WAVES");
+  const char* w = debugEnv("D3D_CONV_WAVES");
   return v | ((w && std::atoi(w) == 4) ? (1 << 30) : 0);
 }
 
 // Tuning / test hook: D3D_CONV_STAGED = "off" keeps the register-gather kernels; "MT,WAVES,NS[,1]" picks a
 // configuration of the staged kernel (trailing 1 = weights resident in LDS); unset = heuristic.
 int stagedOverride() {
-  const char* e = std::getenv("D3D_CONV_STAGED");
+  const char* e = debugEnv("D3D_CONV_STAGED");
   if (!e || !*e) return 0;
   if (std::strcmp(e, "off") == 0) return -1;
   int mt = 0, waves = 0, ns = 0, res = 0;
@@ -521,7 +522,9 @@ struct MMPlugin final : d3d_plugin {
   size_t weightOffset = kMMHeader;             // byte offset of W in blob
   std::shared_ptr<MMDeviceWeights> dev;        // shared by clones (mm_trt.cu:43-45, :75-79)
   std::shared_ptr<std::mutex> devMutex;
-  std::shared_ptr<DeviceBuffer> lastTable;     // keeps the table of the last enqueue alive
+  std::shared_ptr<RulebookLink> linked;        // by-products of the rulebook operator this node is linked to
+  std::shared_ptr<DeviceBuffer> derived;       // neighbour table derived from the index tensor (no link, foreign
+                                               // tensor, inverse)
   std::shared_ptr<DeviceBuffer> widened;       // input rows widened to the MFMA channel count (narrow layers)
 
   static int32_t parse(const void* data, size_t len, MMPlugin** out) {
@@ -578,7 +581,8 @@ struct MMPlugin final : d3d_plugin {
 
   d3d_plugin* clone() const override {
     auto* c = new MMPlugin(*this);  // weights are shared (mm_trt.cu:75-79); per-enqueue buffers are not
-    c->lastTable.reset();
+    c->linked.reset();
+    c->derived.reset();
     c->widened.reset();
     return c;
   }
@@ -613,9 +617,30 @@ struct MMPlugin final : d3d_plugin {
       setError("SPConvMM: feature dtype %d not implemented", dtype);
       return D3D_ERR_UNSUPPORTED;
     }
-    std::lock_guard<std::mutex> lock(*devMutex);
-    if (dev->dtype == dtype) return D3D_OK;
-    if (dtype == D3D_INT8) return configureInt8();
+    {
+      std::lock_guard<std::mutex> lock(*devMutex);
+      if (dev->dtype != dtype) {
+        const int32_t rc = dtype == D3D_INT8 ? configureInt8() : configureFloat(dtype);
+        if (rc != D3D_OK) return rc;
+      }
+    }
+    // Capacities are known here: reserve what enqueue would otherwise have to allocate on first use - the rows of a
+    // narrow layer widened to the MFMA channel count, and the derived table of a node that has no link (or is an
+    // inverse convolution, whose table is always derived).
+    if (in[0].nb_dims == 2 && in[0].dims[0] > 0 && dev->cinMfma > cin) {
+      if (!widened) widened = std::make_shared<DeviceBuffer>();
+      const int32_t rc = widened->reserve(static_cast<size_t>(in[0].dims[0]) * dev->cinMfma * dtypeBytes(dtype));
+      if (rc != D3D_OK) return rc;
+    }
+    if ((!linked || inverse) && maxNumActOut > 0) {
+      if (!derived) derived = std::make_shared<DeviceBuffer>();
+      const int32_t rc = derived->reserve(static_cast<size_t>(kernelVol) * static_cast<size_t>(maxNumActOut) * sizeof(int32_t));
+      if (rc != D3D_OK) return rc;
+    }
+    return D3D_OK;
+  }
+
+  int32_t configureFloat(int32_t dtype) {
     const size_t nW = static_cast<size_t>(kernelVol) * cin * cout;
     std::vector<float> w(nW), b(withBias ? cout : 0);
     std::memcpy(w.data(), blob.data() + weightOffset, nW * 4);
@@ -755,11 +780,28 @@ struct MMPlugin final : d3d_plugin {
     }
     const int64_t rowLen = inDesc[3].dims[1];  // numIndicesMax, mm_trt.cu:169
     const int64_t outRows = outDesc[0].dims[0];
-    std::shared_ptr<DeviceBuffer> table;
-    int32_t rc = neighbourTable(static_cast<const int32_t*>(inputs[3]), rowLen, static_cast<const int32_t*>(inputs[4]),
-                                inverse, kernelVol, outRows, stream, &table);
-    if (rc != D3D_OK) return rc;
-    lastTable = table;
+    const int32_t* nbr = nullptr;
+    const unsigned long long* masks = nullptr;
+    std::shared_ptr<RulebookLink> held = linked;  // by-products are read by the kernels launched below
+    if (held && !inverse) {
+      std::lock_guard<std::mutex> lock(held->mutex);
+      if (held->tableValid && held->index == inputs[3] && held->numIndex == inputs[4] && held->kVol == kernelVol &&
+          held->outRows == outRows && held->rowLen == rowLen) {
+        nbr = static_cast<const int32_t*>(held->table.ptr);
+        if (held->masksValid) masks = static_cast<const unsigned long long*>(held->masks.ptr);
+      }
+    }
+    int32_t rc = D3D_OK;
+    if (!nbr) {  // the index tensor is all there is to go by: derive the table from it
+      if (!derived) derived = std::make_shared<DeviceBuffer>();
+      const size_t bytes = static_cast<size_t>(kernelVol) * static_cast<size_t>(outRows > 0 ? outRows : 1) * sizeof(int32_t);
+      rc = derived->reserve(bytes);
+      if (rc != D3D_OK) return rc;
+      rc = launchBuildNeighbours(static_cast<const int32_t*>(inputs[3]), rowLen, static_cast<const int32_t*>(inputs[4]),
+                                 inverse, kernelVol, outRows, static_cast<int32_t*>(derived->ptr), stream);
+      if (rc != D3D_OK) return rc;
+      nbr = static_cast<const int32_t*>(derived->ptr);
+    }
     const void* zeros = zeroRow();
     ConvArgs a{};
     a.dtype = dtype;
@@ -770,7 +812,7 @@ struct MMPlugin final : d3d_plugin {
     a.outRows = outRows;
     a.in = inputs[0];
     if (dev->cinMfma > cin && (dtype == D3D_INT8 || ((reinterpret_cast<uintptr_t>(outputs[0]) & 15) == 0 &&
-                                                     std::getenv("D3D_CONV_NO_PAD") == nullptr))) {  // narrow layer: widen the rows, then MFMA
+                                                     debugEnv("D3D_CONV_NO_PAD") == nullptr))) {  // narrow layer: widen the rows, then MFMA
       if (!widened) widened = std::make_shared<DeviceBuffer>();
       const int es = dtypeBytes(dtype);
       rc = widened->reserve(static_cast<size_t>(a.inRows > 0 ? a.inRows : 1) * dev->cinMfma * es);
@@ -785,18 +827,11 @@ struct MMPlugin final : d3d_plugin {
     a.weightsMfma = dev->mfma.ptr;
     a.bias = (withBias || dtype == D3D_INT8) ? static_cast<const float*>(dev->bias.ptr) : nullptr;
     a.requantM = dtype == D3D_INT8 ? static_cast<const float*>(dev->requantM.ptr) : nullptr;
-    a.nbr = static_cast<const int32_t*>(table->ptr);
+    a.nbr = nbr;
+    a.tileMasks = masks;
     a.relu = relu ? 1 : 0;
     a.zeros = zeros;
-    if (std::getenv("D3D_TMP_MASKS") && kernelVol <= 64) {  // experiment: masks from a kernel of their own
-      static DeviceBuffer tmpMasks;
-      rc = tmpMasks.reserve(static_cast<size_t>((outRows + 63) / 64 + 1) * 8);
-      if (rc != D3D_OK) return rc;
-      rc = launchTileMasks(a.nbr, outRows, 0, kernelVol, outRows, a.inRows, static_cast<unsigned long long*>(tmpMasks.ptr), stream);
-      if (rc != D3D_OK) return rc;
-      a.tileMasks = static_cast<const unsigned long long*>(tmpMasks.ptr);
-    }
-    if (const char* e = std::getenv("D3D_CONV_PIPE")) a.pipe = e[0] == '0' ? -1 : 0;
+    if (const char* e = debugEnv("D3D_CONV_PIPE")) a.pipe = e[0] == '0' ? -1 : 0;
     a.tileRows = tileRowsOverride();
     a.staged = stagedOverride();
     return launchConv(a, stream);
@@ -1182,9 +1217,39 @@ const char* d3d_last_error(void) { return lastError(); }
 int32_t d3d_num_ops(void) { return static_cast<int32_t>(sizeof(kOps) / sizeof(kOps[0])); }
 const char* d3d_op_name(int32_t i) { return (i >= 0 && i < d3d_num_ops()) ? kOps[i].name : ""; }
 
-void d3d_clear_cache(void) {
-  std::lock_guard<std::mutex> lock(g_cacheMutex);
-  g_cache.clear();
+int32_t d3d_link_rulebook(d3d_plugin* mm, d3d_plugin* idx) {
+  D3D_GUARD_BEGIN
+  auto* m = dynamic_cast<MMPlugin*>(mm);
+  if (!m) {
+    setError("d3d_link_rulebook: the first handle must be an SPConvMM");
+    return D3D_ERR_BAD_ARG;
+  }
+  if (!idx) {
+    m->linked.reset();
+    return D3D_OK;
+  }
+  auto* r = dynamic_cast<IdxPlugin*>(idx);
+  if (!r) {
+    setError("d3d_link_rulebook: the second handle must be an SPConvIdx{N}d");
+    return D3D_ERR_BAD_ARG;
+  }
+  if (r->kVol() != m->kernelVol) {
+    setError("d3d_link_rulebook: kernel volume %d of the convolution, %d of the rulebook", m->kernelVol, r->kVol());
+    return D3D_ERR_BAD_ARG;
+  }
+  // tile masks are read by the kernels of layers with at least 32 (widened) input channels
+  int32_t rc = r->wantByProducts(m->cin > 16);
+  if (rc != D3D_OK) return rc;
+  m->linked = r->link;
+  return D3D_OK;
+  D3D_GUARD_END(D3D_ERR_BAD_ARG)
+}
+
+int32_t d3d_set_option(d3d_plugin* p, int32_t option, int64_t value) {
+  D3D_GUARD_BEGIN
+  if (!p) return D3D_ERR_BAD_ARG;
+  return p->setOption(option, value);
+  D3D_GUARD_END(D3D_ERR_BAD_ARG)
 }
 
 }  // extern "C"

@@ -175,24 +175,36 @@ __device__ __forceinline__ uint32_t blockExclusiveScan(uint32_t v, uint32_t* scr
 // pass of 16-byte stores (replaces resetHashKernel + the cudaMemsetAsync calls
 // of trt/spconv/index.cu:309-314, :352-354).
 // ---------------------------------------------------------------------------
+// Every pass starts with one of the two reset kernels; besides their own clearing they zero the tile masks of
+// the pass and hand the fill state over: fillState[0] (the end of what the previous pass used of the index
+// tensor) takes the value the previous pass left in fillState[1].
+__device__ __forceinline__ void resetShared(int64_t tid, int64_t stride, unsigned long long* masks, int64_t nMasks,
+                                            uint32_t* fillState) {
+  for (int64_t i = tid; i < nMasks; i += stride) masks[i] = 0ull;
+  if (tid == 0 && fillState) fillState[0] = fillState[1];
+}
+
 __global__ void __launch_bounds__(kRbThreads)
 rbReset(uint4* table16, int64_t nTable16, int32_t* index, int64_t nIndex, uint32_t* totals, int kVol,
-        int32_t* numIndex) {
+        int32_t* numIndex, unsigned long long* masks, int64_t nMasks, uint32_t* fillState) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  resetShared(tid, stride, masks, nMasks, fillState);
   const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
   for (int64_t i = tid; i < nTable16; i += stride) table16[i] = ones;
   // index tensor: 16-byte body when the base is aligned, scalar head/tail otherwise
   const uintptr_t base = reinterpret_cast<uintptr_t>(index);
   int64_t head = ((16 - (base & 15)) & 15) >> 2;
   if (head > nIndex) head = nIndex;
-  const int64_t body16 = (nIndex - head) >> 2;
+  const int64_t body16 = index ? (nIndex - head) >> 2 : 0;
   uint4* body = reinterpret_cast<uint4*>(index + head);
   for (int64_t i = tid; i < body16; i += stride) body[i] = ones;
   const int64_t tailStart = head + (body16 << 2);
-  if (tid < head) index[tid] = -1;
-  if (tid < nIndex - tailStart) index[tailStart + tid] = -1;
-  if (tid < kVol) totals[tid] = 0;
+  if (index) {
+    if (tid < head) index[tid] = -1;
+    if (tid < nIndex - tailStart) index[tailStart + tid] = -1;
+  }
+  for (int64_t q = tid; q < kVol; q += stride) totals[q] = 0;
   if (tid == 0) *numIndex = 0;
 }
 
@@ -230,13 +242,28 @@ __device__ __forceinline__ bool tapTarget(const RbGeom& g, const int c[5], const
   return ok;
 }
 
-// Publishes the number of flagged items of this workgroup for its tap.
+// Pairs per tap are kept as kTotalSlots partial sums, totals[tap * kTotalSlots + slot]: atomics on one address are
+// performed one after the other (about 18 ns each across the XCDs), and a pass whose every workgroup adds to the
+// one word of its tap spends longer queueing there than working (1 400 workgroups: 25 us).
+constexpr int kTotalSlots = 8;
+
+__device__ __forceinline__ uint32_t tapPairs(const uint32_t* __restrict__ totals, int tap) {
+  const uint4 a = *reinterpret_cast<const uint4*>(totals + tap * kTotalSlots);
+  const uint4 b = *reinterpret_cast<const uint4*>(totals + tap * kTotalSlots + 4);
+  return a.x + a.y + a.z + a.w + b.x + b.y + b.z + b.w;
+}
+__device__ __forceinline__ uint32_t tapSegment(const uint32_t* __restrict__ totals, int tap) {
+  return (tapPairs(totals, tap) + (kSegment - 1)) & ~static_cast<uint32_t>(kSegment - 1);
+}
+
+// Publishes the number of flagged items of this workgroup for its tap; `slots` = kTotalSlots for the pair totals,
+// 1 for a plain array of per-tap sums.
 __device__ __forceinline__ void publishCount(uint32_t mine, uint32_t* scratch, uint32_t* cnt, uint32_t nBlocks,
-                                             uint32_t* totals) {
+                                             uint32_t* totals, int slots) {
   const uint32_t total = blockSum(mine, scratch);
   if (threadIdx.x == 0) {
     cnt[static_cast<size_t>(blockIdx.y) * nBlocks + blockIdx.x] = total;
-    if (total) atomicAdd(&totals[blockIdx.y], total);
+    if (total) atomicAdd(&totals[blockIdx.y * slots + blockIdx.x % slots], total);
   }
 }
 
@@ -280,10 +307,10 @@ rbSubmProbe(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restri
       }
       found += row[j] != kNone;
     }
-    if (first < n) *reinterpret_cast<uint4*>(staging + static_cast<size_t>(tap) * pitch + first) =
+    if (first < n) *reinterpret_cast<uint4*>(staging + static_cast<int64_t>(tap) * pitch + first) =
         make_uint4(row[0], row[1], row[2], row[3]);
   }
-  publishCount(found, scratch, cnt, nBlocks, totals);
+  publishCount(found, scratch, cnt, nBlocks, totals, kTotalSlots);
 }
 
 // ---------------------------------------------------------------------------
@@ -313,7 +340,7 @@ rbConvInsert(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restr
         slot[j] = hashInsertMin(table, mask, off, static_cast<uint32_t>(i) * static_cast<uint32_t>(g.kVol) + tap);
     }
   }
-  *reinterpret_cast<uint4*>(staging + static_cast<size_t>(tap) * pitch + first) =
+  *reinterpret_cast<uint4*>(staging + static_cast<int64_t>(tap) * pitch + first) =
       make_uint4(slot[0], slot[1], slot[2], slot[3]);
 }
 
@@ -323,7 +350,7 @@ __device__ __forceinline__ void loadOwned(const RbGeom& g, int n, int tap, int64
                                           const uint32_t* __restrict__ staging, uint32_t slot[kRbItems],
                                           unsigned long long entry[kRbItems], bool own[kRbItems]) {
   uint4 s4 = make_uint4(kNone, kNone, kNone, kNone);
-  if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<size_t>(tap) * pitch + first);
+  if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<int64_t>(tap) * pitch + first);
   slot[0] = s4.x; slot[1] = s4.y; slot[2] = s4.z; slot[3] = s4.w;
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
@@ -354,7 +381,7 @@ rbConvOwner(RbGeom g, const int32_t* __restrict__ numActIn, int64_t cap, int64_t
 #pragma unroll
     for (int j = 0; j < kRbItems; ++j) mine += own[j];
   }
-  publishCount(mine, scratch, ownCnt, nBlocks, ownTotals);
+  publishCount(mine, scratch, ownCnt, nBlocks, ownTotals, 1);
 }
 
 // Pass 3: output rows are numbered in (tap, owner input row) order; writes the
@@ -425,7 +452,7 @@ rbConvResolve(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, 
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
   uint32_t found = 0;
   if (first < n) {
-    uint4* cell = reinterpret_cast<uint4*>(staging + static_cast<size_t>(tap) * pitch + first);
+    uint4* cell = reinterpret_cast<uint4*>(staging + static_cast<int64_t>(tap) * pitch + first);
     const uint4 s4 = *cell;
     uint32_t v[kRbItems] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
@@ -440,7 +467,7 @@ rbConvResolve(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, 
     }
     *cell = make_uint4(v[0], v[1], v[2], v[3]);
   }
-  publishCount(found, scratch, cnt, nBlocks, totals);
+  publishCount(found, scratch, cnt, nBlocks, totals, kTotalSlots);
 }
 
 // ---------------------------------------------------------------------------
@@ -451,23 +478,68 @@ rbConvResolve(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, 
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(kRbThreads)
 rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int kVol,
-          const uint32_t* __restrict__ staging, const uint32_t* __restrict__ cnt, uint32_t nBlocks,
+          const uint32_t* staging, const uint32_t* __restrict__ cnt, uint32_t nBlocks,
           const uint32_t* __restrict__ totals, int32_t* __restrict__ gather, int32_t* __restrict__ scatter,
-          int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* __restrict__ nbr, int64_t nbrRows,
-          const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int mirror) {
+          int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* nbr, int64_t nbrRows,
+          const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int mirror, int inPlace,
+          unsigned long long* __restrict__ masks, uint32_t* fillState, int incrementalFill) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int tap = blockIdx.y;
   const uint32_t b = blockIdx.x;
   if (b == 0 && tap == 0 && threadIdx.x == 0) {
     uint32_t end = 0;
-    for (int t = 0; t < kVol; ++t) end += (totals[t] + (kSegment - 1)) & ~static_cast<uint32_t>(kSegment - 1);
+    for (int t = 0; t < kVol; ++t) end += tapSegment(totals, t);
     *numIndex = static_cast<int32_t>(end);
+    if (fillState) fillState[1] = end;  // what this pass uses of the index tensor: the next pass clears from here
+  }
+  // The index tensor still holds the previous pass (of this operator, at this address): instead of clearing it at
+  // capacity, write -1 where that pass had entries and this one has none - behind the new end up to the old one,
+  // and in the gap that rounds this tap's segment up to 128.  Only the first workgroups of every tap take part
+  // (at least 64 of them when the grid has as many), so the others do not wait for the segment ends; the range
+  // behind the new end is short unless the scene changed a lot between the two passes.
+  const uint32_t fillers = 64u / static_cast<uint32_t>(kVol) + 1u < gridDim.x ? 64u / static_cast<uint32_t>(kVol) + 1u : gridDim.x;
+  if (incrementalFill && b < fillers) {
+    uint32_t end = 0, myStart = 0;
+    for (int t = 0; t < kVol; ++t) {
+      if (t == tap) myStart = end;
+      end += tapSegment(totals, t);
+    }
+    const uint32_t oldEnd = fillState[0];
+    const uint32_t gid = (static_cast<uint32_t>(tap) * fillers + b) * kRbThreads + threadIdx.x;
+    const uint32_t nThreads = fillers * gridDim.y * kRbThreads;
+    // segment ends are multiples of 128 entries: 16-byte stores when the three rows are 16-byte aligned
+    if (((reinterpret_cast<uintptr_t>(gather) | reinterpret_cast<uintptr_t>(scatter) |
+          reinterpret_cast<uintptr_t>(tapRow)) & 15) == 0) {
+      const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
+      for (uint32_t i = end / 4 + gid; i < oldEnd / 4; i += nThreads) {
+        reinterpret_cast<uint4*>(gather)[i] = ones;
+        reinterpret_cast<uint4*>(scatter)[i] = ones;
+        reinterpret_cast<uint4*>(tapRow)[i] = ones;
+      }
+    } else {
+      for (uint32_t i = end + gid; i < oldEnd; i += nThreads) {
+        gather[i] = -1;
+        scatter[i] = -1;
+        tapRow[i] = -1;
+      }
+    }
+    if (b == 0 && threadIdx.x < kSegment) {
+      const uint32_t i = myStart + tapPairs(totals, tap) + threadIdx.x;
+      if (i < myStart + tapSegment(totals, tap)) {
+        gather[i] = -1;
+        scatter[i] = -1;
+        tapRow[i] = -1;
+      }
+    }
   }
   const int n = liveCount(numActIn, cap);
   const int64_t first = static_cast<int64_t>(b) * kRbChunk + threadIdx.x * kRbItems;
   // Mirror mode (SubM with "same" padding): the pair (tap, in i -> out o) has the twin (kVol-1-tap, in o -> out i),
   // so row i of the neighbour table under the mirrored tap is simply o - this thread's own staging entry.  The
-  // table is then written here in whole coalesced rows, -1 included: no fill pass, no scatter.
+  // table is then written here in whole coalesced rows, -1 included: no fill pass, no scatter.  With inPlace the
+  // probe pass already used the table rows as its staging rows (staging + tap * pitch IS the row below): only
+  // what the probe did not leave right is stored - entries of rows past the live count, and rows where ranks have
+  // to become row numbers.
   int32_t* nbrRow = (mirror && nbr) ? nbr + static_cast<int64_t>(kVol - 1 - tap) * nbrRows : nullptr;
   auto mirrorStore = [&](const uint32_t (&o)[kRbItems]) {
     if (!nbrRow) return;
@@ -485,26 +557,37 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
     return;
   }
 
+  // the staging entries first: their latency overlaps that of the sums below
+  uint4 s4 = make_uint4(kNone, kNone, kNone, kNone);
+  if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<int64_t>(tap) * pitch + first);
   uint32_t before = 0;
   for (uint32_t q = threadIdx.x; q < b; q += blockDim.x) before += cnt[static_cast<size_t>(tap) * nBlocks + q];
   uint32_t pos = blockSum(before, scratch);
-  for (int t = 0; t < tap; ++t) pos += (totals[t] + (kSegment - 1)) & ~static_cast<uint32_t>(kSegment - 1);
+  for (int t = 0; t < tap; ++t) pos += tapSegment(totals, t);
 
-  uint4 s4 = make_uint4(kNone, kNone, kNone, kNone);
-  if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<size_t>(tap) * pitch + first);
   uint32_t v[kRbItems] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j)
     if (first + j >= n) v[j] = kNone;
-  if (perm && *permShuffled) {  // block-map SubM: the probe stored ranks; rows are perm[rank]
+  const bool shuffled = perm && *permShuffled;
+  if (shuffled) {  // block-map SubM: the probe stored ranks; rows are perm[rank]
 #pragma unroll
     for (int j = 0; j < kRbItems; ++j)
       if (v[j] != kNone) v[j] = perm[v[j]];
   }
-  mirrorStore(v);
+  if (!inPlace || shuffled || first + kRbItems > n) mirrorStore(v);
   uint32_t mine = 0;
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) mine += (v[j] != kNone);
+  if (masks && mirror && kVol <= 64) {
+    // tile masks of the convolution (bit t of masks[r / 64]: some output row of 64-row tile r / 64 has tap t).
+    // Mirrored table: this thread's 4 consecutive INPUT rows are output rows under tap kVol-1-tap; a 16-lane row
+    // covers exactly one tile.
+    const unsigned long long any = __ballot(mine != 0);
+    const int lane = threadIdx.x & 63;
+    if ((lane & 15) == 0 && ((any >> lane) & 0xFFFFull) && first < nbrRows)
+      atomicOr(&masks[first >> 6], 1ull << (kVol - 1 - tap));
+  }
   uint32_t total;
   uint32_t at = pos + blockExclusiveScan(mine, scratch, &total);
 #pragma unroll
@@ -601,9 +684,10 @@ __device__ __forceinline__ void fillMinusOneRange(int32_t* p, int64_t n, int64_t
 
 __global__ void __launch_bounds__(kRbThreads)
 bmReset(uint4* records16, int64_t nRecords, int32_t* index, int64_t nIndex, uint32_t* counters, int64_t nCounters,
-        int32_t* numIndex) {
+        int32_t* numIndex, unsigned long long* masks, int64_t nMasks, uint32_t* fillState) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  resetShared(tid, stride, masks, nMasks, fillState);
   const uint4 zero = make_uint4(0, 0, 0, 0);
   for (int64_t i = tid; i < nRecords; i += stride) records16[i] = zero;
   fillMinusOneRange(index, nIndex, tid, stride);  // index == nullptr: a later pass fills it
@@ -857,10 +941,10 @@ bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* 
       }
       found += row[j] != kNone;
     }
-    if (first < n) *reinterpret_cast<uint4*>(staging + static_cast<size_t>(tap) * pitch + first) =
+    if (first < n) *reinterpret_cast<uint4*>(staging + static_cast<int64_t>(tap) * pitch + first) =
         make_uint4(row[0], row[1], row[2], row[3]);
   }
-  publishCount(found, scratch, cnt, nBlocks, totals);
+  publishCount(found, scratch, cnt, nBlocks, totals, kTotalSlots);
 }
 
 // ---------------------------------------------------------------------------
@@ -1123,7 +1207,7 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
         }
       }
     }
-    if (live) staging[static_cast<size_t>(tap) * pitch + i] = row;
+    if (live) staging[static_cast<int64_t>(tap) * pitch + i] = row;
     const uint32_t hits = static_cast<uint32_t>(__popcll(__ballot(row != kNone)));
     if (KSEL != 0) {
       if (lane == tap) mine += hits;           // tap is a compile-time constant below 64 here
@@ -1138,7 +1222,132 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
     const uint32_t v = ldsCnt[t];
     if (v) {
       atomicAdd(&cnt[static_cast<size_t>(t) * nBlocks + chunk], v);
-      atomicAdd(&totals[t], v);
+      atomicAdd(&totals[t * kTotalSlots + probeBlock % kTotalSlots], v);
+    }
+  }
+}
+
+// The same pass for the kernel shapes of fixedKernelShape (3-D, dilation 1, strides 1 / 2 / 4, not transposed),
+// with K1 threads per input: thread (i, i1) resolves the K2*K3 taps of kernel position i1 along the outermost
+// dim.  A brick is one level of that dim, so these taps look into the 2x2 bricks of ONE level: 4 record loads and
+// 64 bytes of LDS per thread instead of 12 and 192, three times the threads - the pass is bound by the latency
+// of its dependent accesses, and this is what hides it.  Workgroup roles by block index: first the fill
+// workgroups (-1 over the neighbour table, bandwidth-bound work beside latency-bound work), then
+// K1 * probeBlocks probing workgroups (the K1 of one 256-input block next to each other), then the pass only
+// the compaction waits for (rank -> row permutation, or the output coordinates).
+template <bool SUBM, int K1, int K2, int K3>
+__global__ void __launch_bounds__(kRbThreads)
+bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
+             int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+             uint32_t* __restrict__ perm, uint32_t* permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
+             uint32_t* cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
+             int64_t nFillB, uint32_t fillBlocks, uint32_t probeBlocks, int32_t* __restrict__ outCoors,
+             uint32_t nRecords) {
+  constexpr int KP = K2 * K3;
+  __shared__ uint4 group[4 * kRbThreads];
+  __shared__ uint32_t ldsCnt[KP];
+  if (blockIdx.x < fillBlocks) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * kRbThreads + threadIdx.x;
+    const int64_t stride = static_cast<int64_t>(fillBlocks) * kRbThreads;
+    fillMinusOneRange(fillA, nFillA, tid, stride);
+    fillMinusOneRange(fillB, nFillB, tid, stride);
+    return;
+  }
+  const uint32_t pidx = blockIdx.x - fillBlocks;
+  if (pidx >= probeBlocks * K1) {
+    const uint32_t e = pidx - probeBlocks * K1;
+    if (SUBM) {
+      permuteRow(g, m, coors, liveCount(numActIn, cap), static_cast<int64_t>(e) * kRbThreads + threadIdx.x, records,
+                 chunkBase, perm, permShuffled);
+    } else {
+      emitRecordCoords(g, m, records, chunkBase, nRecords, e * (kRbThreads / 64) + (threadIdx.x >> 6), outCoors,
+                       maxNumActOut);
+    }
+    return;
+  }
+  const int i1 = static_cast<int>(pidx % K1);
+  const uint32_t probeBlock = pidx / K1;
+  const int n = liveCount(numActIn, cap);
+  const int64_t i0 = static_cast<int64_t>(probeBlock) * kRbThreads;
+  if (i0 >= n) return;  // workgroup-uniform
+  if (threadIdx.x < KP) ldsCnt[threadIdx.x] = 0;
+  const int64_t i = i0 + threadIdx.x;
+  const bool live = i < n;
+  int c[5] = {0, 0, 0, 0, 0};
+  if (live) loadCoord(coors, g.nd, i, c);  // (b, z, y, x) in c[0], c[2..4]; c[1] is the degenerate dim
+  // per dim and kernel position: validity, brick, cell inside the brick
+  auto along = [&](int dim, int pos, int* brick, uint32_t* part) {
+    const int st = g.s[dim];
+    const int ls = st >> 1 > 1 ? 2 : st >> 1;
+    const int num = c[dim + 1] + g.p[dim] - pos;
+    const int o = num >> ls;
+    *brick = o >> m.shift[dim];
+    *part = static_cast<uint32_t>(o) & ((1u << m.shift[dim]) - 1);
+    return num >= 0 && (num & (st - 1)) == 0 && o < g.shape[dim + 1];
+  };
+  int brick1;
+  uint32_t part1;
+  const bool ok1 = along(1, i1, &brick1, &part1) && live && c[0] >= 0 && c[0] < g.shape[0] && c[1] == 0;
+  bool ok2[K2], ok3[K3];
+  int b2[K2], b3[K3];
+  uint32_t part2[K2], part3[K3];
+#pragma unroll
+  for (int q = 0; q < K2; ++q) ok2[q] = along(2, q, &b2[q], &part2[q]);
+#pragma unroll
+  for (int q = 0; q < K3; ++q) ok3[q] = along(3, q, &b3[q], &part3[q]);
+  // lower brick of the 2x2 group per dim: that of the highest kernel position (the lowest cell), clamped to 0
+  const int base2 = b2[K2 - 1] > 0 ? b2[K2 - 1] : 0, base3 = b3[K3 - 1] > 0 ? b3[K3 - 1] : 0;
+  const uint32_t rec0 = ((static_cast<uint32_t>(ok1 ? c[0] : 0) * static_cast<uint32_t>(m.nb[0])) *
+                             static_cast<uint32_t>(m.nb[1]) + static_cast<uint32_t>(ok1 ? brick1 : 0)) *
+                            static_cast<uint32_t>(m.nb[2]) * static_cast<uint32_t>(m.nb[3]);
+  uint4 loaded[4];
+  uint32_t base[4];
+  bool present[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int y = base2 + (e >> 1), x = base3 + (e & 1);
+    present[e] = ok1 && y < m.nb[2] && x < m.nb[3];
+    const uint32_t rec = present[e] ? rec0 + static_cast<uint32_t>(y * m.nb[3] + x) : 0u;
+    loaded[e] = *reinterpret_cast<const uint4*>(records + rec);
+    base[e] = chunkBase[rec / kRbChunk];
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    loaded[e].z += base[e];  // in-chunk prefix -> global prefix
+    group[e * kRbThreads + threadIdx.x] = present[e] ? loaded[e] : make_uint4(0, 0, 0, 0);
+  }
+  __syncthreads();  // ldsCnt zeroed
+  uint32_t mine = 0;  // lane t of a wavefront counts the wavefront's pairs of tap i1 * KP + t
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int q2 = 0; q2 < K2; ++q2)
+#pragma unroll
+    for (int q3 = 0; q3 < K3; ++q3) {
+      uint32_t row = kNone;
+      if (ok1 && ok2[q2] && ok3[q3]) {
+        const int member = (((b2[q2] - base2) & 1) << 1) | ((b3[q3] - base3) & 1);
+        const uint4 v = group[member * kRbThreads + threadIdx.x];
+        const unsigned long long bits = (static_cast<unsigned long long>(v.y) << 32) | v.x;
+        const uint32_t bit = (((part1 << m.shift[2]) | part2[q2]) << m.shift[3]) | part3[q3];
+        if ((bits >> bit) & 1ull) {
+          const uint32_t rank = v.z + static_cast<uint32_t>(__popcll(bits & ((1ull << bit) - 1ull)));
+          if (SUBM || rank < static_cast<uint32_t>(maxNumActOut)) row = rank;
+        }
+      }
+      const int tap = (i1 * K2 + q2) * K3 + q3;
+      if (live) staging[static_cast<int64_t>(tap) * pitch + i] = row;
+      const uint32_t hits = static_cast<uint32_t>(__popcll(__ballot(row != kNone)));
+      if (lane == q2 * K3 + q3) mine += hits;
+    }
+  if (mine) atomicAdd(&ldsCnt[lane], mine);
+  __syncthreads();
+  const uint32_t chunk = probeBlock / kRbItems;
+  if (threadIdx.x < KP) {
+    const uint32_t v = ldsCnt[threadIdx.x];
+    if (v) {
+      const int tap = i1 * KP + threadIdx.x;
+      atomicAdd(&cnt[static_cast<size_t>(tap) * nBlocks + chunk], v);
+      atomicAdd(&totals[tap * kTotalSlots + probeBlock % kTotalSlots], v);
     }
   }
 }
@@ -1190,7 +1399,7 @@ constexpr uint64_t kMaxBlockMapBytes = 256ull << 20;
 // D3D_RULEBOOK=hash or =blockmap pins the occupancy structure (tests, tuning);
 // otherwise the block map is used whenever its records fit kMaxBlockMapBytes.
 int structureOverride() {
-  const char* e = std::getenv("D3D_RULEBOOK");
+  const char* e = debugEnv("D3D_RULEBOOK");
   if (!e) return 0;
   if (std::strcmp(e, "hash") == 0) return 1;
   if (std::strcmp(e, "blockmap") == 0) return 2;
@@ -1198,6 +1407,9 @@ int structureOverride() {
 }
 
 size_t scanGroups(uint32_t nChunks) { return (static_cast<size_t>(nChunks) + kScanGroup - 1) / kScanGroup; }
+size_t totalsWords(int kVol, uint32_t nChunks) {
+  return static_cast<size_t>(kVol) * (kTotalSlots + 1) + 2 + scanGroups(nChunks);
+}
 
 RbWorkspace planWith(const RbGeom& g, int64_t cap, bool subM, bool blockMap) {
   RbWorkspace w{};
@@ -1241,11 +1453,11 @@ RbWorkspace planWith(const RbGeom& g, int64_t cap, bool subM, bool blockMap) {
   }
   w.staging = off;
   off = alignUp(off + static_cast<size_t>(g.kVol) * w.pitch * 4);
-  w.cnt = off;     // [kVol, nBlocks], directly followed (no gap) by
-  off += static_cast<size_t>(g.kVol) * w.nBlocks * 4;
-  w.totals = off;  // [2, kVol] + 2 + groups: valid pairs per tap, owned outputs per tap, "rows not in rank order" flag,
-                   // scan ticket, first-level scan tickets
-  off = alignUp(off + (static_cast<size_t>(g.kVol) * 2 + 2 + scanGroups(w.nChunks)) * 4);
+  w.cnt = off;     // [kVol, nBlocks], followed (the counters are cleared as one range) by
+  off = alignUp(off + static_cast<size_t>(g.kVol) * w.nBlocks * 4, 16);
+  w.totals = off;  // [kVol, kTotalSlots] valid pairs per tap in partial sums, [kVol] owned outputs per tap, "rows not
+                   // in rank order" flag, scan ticket, first-level scan tickets
+  off = alignUp(off + totalsWords(g.kVol, w.nChunks) * 4);
   w.total = off;
   return w;
 }
@@ -1257,14 +1469,14 @@ bool nearEligible(const RbGeom& g, const BlockMap& m) {
     const int reach = g.transpose ? (g.k[dim] - 1) * g.d[dim] : ((g.k[dim] - 1) * g.d[dim]) / g.s[dim];
     if (reach > ((kNearMembers[dim] - 1) << m.shift[dim])) return false;
   }
-  const char* e = std::getenv("D3D_RULEBOOK_NEAR");
+  const char* e = debugEnv("D3D_RULEBOOK_NEAR");
   return !(e && e[0] == '0');
 }
 
 // 1: 3x3x3, 2: 3x1x1, 3: 3x1x3, 4: 1x3x3 (3-D, dilation 1, strides 1/2/4, not transposed), else 0 = general code.
 // D3D_RULEBOOK_FIXED=0 forces the general enumeration (tests).
 int fixedKernelShape(const RbGeom& g) {
-  const char* e = std::getenv("D3D_RULEBOOK_FIXED");
+  const char* e = debugEnv("D3D_RULEBOOK_FIXED");
   if (e && e[0] == '0') return 0;
   if (g.nd != 3 || g.transpose || g.k[0] != 1) return 0;
   for (int dim = 1; dim < kMaxSpatial; ++dim)
@@ -1306,7 +1518,15 @@ RbWorkspace planRulebookWorkspace(const RbGeom& g, int64_t cap, bool subM, size_
 
 int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const int32_t* numActIn, int64_t cap,
                        int32_t maxNumActOut, int32_t* index, int32_t* numIndex, int32_t* outCoors, int32_t* numActOut,
-                       void* workspace, size_t workspaceBytes, int32_t* nbrOut, int64_t nbrRows, hipStream_t stream) {
+                       void* workspace, size_t workspaceBytes, RbSide& side, hipStream_t stream) {
+  side.masksWritten = false;
+  int32_t* const nbrOut = side.nbrRows > 0 ? side.nbr : nullptr;
+  const int64_t nbrRows = nbrOut ? side.nbrRows : 0;
+  // tile masks go with the table; the fill state lets this pass clear only what the previous one left behind
+  unsigned long long* masks = (nbrOut && g.kVol <= 64) ? side.masks : nullptr;
+  uint32_t* const fillState = side.fillState;
+  const bool incremental = side.incrementalFill && fillState;
+  int32_t* const fillIndex = incremental ? nullptr : index;
   if (!coors || !numActIn || !index || !numIndex || (!subM && (!outCoors || !numActOut))) {
     setError("rulebook: null tensor pointer");
     return D3D_ERR_BAD_ARG;
@@ -1341,10 +1561,11 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     return D3D_ERR_BAD_ARG;
   }
   char* ws = static_cast<char*>(workspace);
-  auto* staging = reinterpret_cast<uint32_t*>(ws + w.staging);
+  uint32_t* staging = reinterpret_cast<uint32_t*>(ws + w.staging);
+  int64_t pitch = w.pitch;
   auto* cnt = reinterpret_cast<uint32_t*>(ws + w.cnt);
   auto* totals = reinterpret_cast<uint32_t*>(ws + w.totals);
-  uint32_t* ownTotals = totals + g.kVol;
+  uint32_t* ownTotals = totals + g.kVol * kTotalSlots;
   const int64_t rowLen = static_cast<int64_t>(g.kVol) * (cap + kSegment);
   const int64_t nIndex = 3 * rowLen;
   const dim3 block(kRbThreads);
@@ -1363,9 +1584,23 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   for (int dim = 0; dim < kMaxSpatial; ++dim)
     if (g.s[dim] != 1 || 2 * g.p[dim] != (g.k[dim] - 1) * g.d[dim]) mirror = false;
   {
-    const char* e = std::getenv("D3D_RULEBOOK_MIRROR");
+    const char* e = debugEnv("D3D_RULEBOOK_MIRROR");
     if (e && e[0] == '0') mirror = false;
   }
+  // Tile masks come with the mirrored table, whose rows are written whole by the lanes that hold them; a scattered
+  // table would need an atomic per pair for them (measured: 18 us on a 640k-pair rulebook, more than the
+  // convolution saves by skipping taps).
+  // The mirrored table's rows are what the probe pass stages (row kVol-1-tap = the output rows of tap's pairs):
+  // with 16-byte aligned rows the probe writes them straight into the table - a base at its last row and a
+  // negative pitch make staging[tap * pitch + i] that entry - and the compaction reads them from there.
+  const bool inPlace = mirror && cap % 4 == 0 && (reinterpret_cast<uintptr_t>(nbrOut) & 15) == 0;
+  if (inPlace) {
+    staging = reinterpret_cast<uint32_t*>(nbrOut) + static_cast<int64_t>(g.kVol - 1) * nbrRows;
+    pitch = -nbrRows;
+  }
+  if (!mirror) masks = nullptr;
+  const int64_t nMasks = masks ? side.nMasks : 0;
+  side.masksWritten = masks != nullptr;
   bool nbrFilled = mirror;
   const uint32_t* compactPerm = nullptr;      // block-map SubM: staging holds ranks, rows = perm[rank] when shuffled
   const uint32_t* compactPermFlag = nullptr;
@@ -1375,9 +1610,9 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     auto* records = reinterpret_cast<BmRecord*>(ws + w.table);
     auto* perm = reinterpret_cast<uint32_t*>(ws + w.ids);
     auto* chunkBase = reinterpret_cast<uint32_t*>(ws + w.ownCnt);
-    uint32_t* scanTicket = totals + 2 * g.kVol + 1;
+    uint32_t* scanTicket = ownTotals + g.kVol + 1;
     const dim3 perChunk(w.nChunks > 0 ? w.nChunks : 1);
-    uint32_t* permShuffled = totals + 2 * g.kVol;
+    uint32_t* permShuffled = ownTotals + g.kVol;
     if (subM) {
       compactPerm = perm;
       compactPermFlag = permShuffled;
@@ -1385,11 +1620,11 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     const bool near = nearEligible(g, m);
     const int ksel = near ? fixedKernelShape(g) : 0;
     const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
-    hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + (near ? 0 : nIndex / 4) + 1), block, 0,
+    hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + ((near || incremental) ? 0 : nIndex / 4) + 1), block, 0,
                        stream, reinterpret_cast<uint4*>(records), static_cast<int64_t>(w.nRecords),
-                       near ? nullptr : index, nIndex, cnt,
-                       static_cast<int64_t>(g.kVol) * w.nBlocks + 2 * g.kVol + 2 + static_cast<int64_t>(scanGroups(w.nChunks)),
-                       numIndex);
+                       near ? nullptr : fillIndex, nIndex, cnt,
+                       static_cast<int64_t>((w.totals - w.cnt) / 4 + totalsWords(g.kVol, w.nChunks)),
+                       numIndex, masks, nMasks, fillState);
     if (subM) {
       hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
     } else if (near) {
@@ -1422,32 +1657,42 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       const int64_t nFillB = fillB ? static_cast<int64_t>(g.kVol) * nbrRows : 0;
       nbrFilled = true;
 #define D3D_LAUNCH_PROBE_NEAR(SUBM, KSEL)                                                                          \
-  hipLaunchKernelGGL((bmProbeNear<SUBM, KSEL>), fused, block, nearLds, stream, g, m, coors, numActIn, cap, w.pitch,   \
-                     records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, index,    \
+  hipLaunchKernelGGL((bmProbeNear<SUBM, KSEL>), fused, block, nearLds, stream, g, m, coors, numActIn, cap, pitch,   \
+                     records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, fillIndex, \
                      nIndex, fillB, nFillB, quads, outCoors, w.nRecords)
+      // fixed kernel shapes: K1 threads per input; fill workgroups only for what there is to fill
+      const int64_t fillItems = (fillIndex ? nIndex : 0) + nFillB;
+      uint32_t planeFill = static_cast<uint32_t>((fillItems / 4 + kRbThreads - 1) / kRbThreads);
+      if (planeFill > 1024) planeFill = 1024;
+#define D3D_LAUNCH_PROBE_PLANE(SUBM, K1, K2, K3)                                                                    \
+  hipLaunchKernelGGL((bmProbePlane<SUBM, K1, K2, K3>), dim3(planeFill + probeBlocks * K1 + extra), block, 0, stream, \
+                     g, m, coors, numActIn, cap, pitch, records, chunkBase, perm, permShuffled, maxNumActOut,     \
+                     staging, cnt, w.nBlocks, totals, fillIndex, nIndex, fillB, nFillB, planeFill, probeBlocks,     \
+                     outCoors, w.nRecords)
       if (subM) {
         switch (ksel) {
-          case 1: D3D_LAUNCH_PROBE_NEAR(true, 1); break;
-          case 2: D3D_LAUNCH_PROBE_NEAR(true, 2); break;
-          case 3: D3D_LAUNCH_PROBE_NEAR(true, 3); break;
-          case 4: D3D_LAUNCH_PROBE_NEAR(true, 4); break;
+          case 1: D3D_LAUNCH_PROBE_PLANE(true, 3, 3, 3); break;
+          case 2: D3D_LAUNCH_PROBE_PLANE(true, 3, 1, 1); break;
+          case 3: D3D_LAUNCH_PROBE_PLANE(true, 3, 1, 3); break;
+          case 4: D3D_LAUNCH_PROBE_PLANE(true, 1, 3, 3); break;
           default: D3D_LAUNCH_PROBE_NEAR(true, 0);
         }
       } else {
         switch (ksel) {
-          case 1: D3D_LAUNCH_PROBE_NEAR(false, 1); break;
-          case 2: D3D_LAUNCH_PROBE_NEAR(false, 2); break;
-          case 3: D3D_LAUNCH_PROBE_NEAR(false, 3); break;
-          case 4: D3D_LAUNCH_PROBE_NEAR(false, 4); break;
+          case 1: D3D_LAUNCH_PROBE_PLANE(false, 3, 3, 3); break;
+          case 2: D3D_LAUNCH_PROBE_PLANE(false, 3, 1, 1); break;
+          case 3: D3D_LAUNCH_PROBE_PLANE(false, 3, 1, 3); break;
+          case 4: D3D_LAUNCH_PROBE_PLANE(false, 1, 3, 3); break;
           default: D3D_LAUNCH_PROBE_NEAR(false, 0);
         }
       }
+#undef D3D_LAUNCH_PROBE_PLANE
 #undef D3D_LAUNCH_PROBE_NEAR
     } else if (subM) {
-      hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, chunkBase, perm,
+      hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, pitch, records, chunkBase, perm,
                          permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
     } else {
-      hipLaunchKernelGGL(bmProbe<false>, perTap, block, 0, stream, g, m, coors, numActIn, cap, w.pitch, records, chunkBase, perm,
+      hipLaunchKernelGGL(bmProbe<false>, perTap, block, 0, stream, g, m, coors, numActIn, cap, pitch, records, chunkBase, perm,
                          permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
     }
   } else {
@@ -1456,29 +1701,30 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     auto* ownCnt = reinterpret_cast<uint32_t*>(ws + w.ownCnt);
     const uint32_t mask = w.slots - 1;
     const int64_t nTable16 = static_cast<int64_t>(w.slots) / 2;
-    hipLaunchKernelGGL(rbReset, fillGrid(nTable16 + nIndex / 4 + 1), block, 0, stream,
-                       reinterpret_cast<uint4*>(table), nTable16, index, nIndex, totals, 2 * g.kVol, numIndex);
+    hipLaunchKernelGGL(rbReset, fillGrid(nTable16 + (incremental ? 0 : nIndex / 4) + 1), block, 0, stream,
+                       reinterpret_cast<uint4*>(table), nTable16, fillIndex, nIndex, totals, g.kVol * (kTotalSlots + 1), numIndex, masks,
+                       nMasks, fillState);
     if (subM) {
       hipLaunchKernelGGL(rbSubmInsert, perInput, block, 0, stream, g, coors, numActIn, cap, table, mask);
-      hipLaunchKernelGGL(rbSubmProbe, perTap, block, 0, stream, g, coors, numActIn, cap, w.pitch, table, mask,
+      hipLaunchKernelGGL(rbSubmProbe, perTap, block, 0, stream, g, coors, numActIn, cap, pitch, table, mask,
                          staging, cnt, w.nBlocks, totals);
     } else {
-      hipLaunchKernelGGL(rbConvInsert, perTap, block, 0, stream, g, coors, numActIn, cap, w.pitch, table, mask,
+      hipLaunchKernelGGL(rbConvInsert, perTap, block, 0, stream, g, coors, numActIn, cap, pitch, table, mask,
                          staging);
-      hipLaunchKernelGGL(rbConvOwner, perTap, block, 0, stream, g, numActIn, cap, w.pitch, table, staging, ownCnt,
+      hipLaunchKernelGGL(rbConvOwner, perTap, block, 0, stream, g, numActIn, cap, pitch, table, staging, ownCnt,
                          w.nBlocks, ownTotals);
-      hipLaunchKernelGGL(rbConvAssign, perTap, block, 0, stream, g, numActIn, cap, w.pitch, table, staging, ownCnt,
+      hipLaunchKernelGGL(rbConvAssign, perTap, block, 0, stream, g, numActIn, cap, pitch, table, staging, ownCnt,
                          w.nBlocks, ownTotals, ids, outCoors, numActOut, maxNumActOut);
-      hipLaunchKernelGGL(rbConvResolve, perTap, block, 0, stream, numActIn, cap, w.pitch, ids, staging, maxNumActOut,
+      hipLaunchKernelGGL(rbConvResolve, perTap, block, 0, stream, numActIn, cap, pitch, ids, staging, maxNumActOut,
                          cnt, w.nBlocks, totals);
     }
   }
   if (nbrOut && nbrRows > 0 && !nbrFilled)
     hipLaunchKernelGGL(rbFillMinusOne, fillGrid(static_cast<int64_t>(g.kVol) * nbrRows / 4 + 1), block, 0, stream, nbrOut,
                        static_cast<int64_t>(g.kVol) * nbrRows);
-  hipLaunchKernelGGL(rbCompact, perTap, block, 0, stream, numActIn, cap, w.pitch, g.kVol, staging, cnt, w.nBlocks,
+  hipLaunchKernelGGL(rbCompact, perTap, block, 0, stream, numActIn, cap, pitch, g.kVol, staging, cnt, w.nBlocks,
                      totals, index, index + rowLen, index + 2 * rowLen, numIndex, nbrRows > 0 ? nbrOut : nullptr, nbrRows,
-                     compactPerm, compactPermFlag, mirror ? 1 : 0);
+                     compactPerm, compactPermFlag, mirror ? 1 : 0, inPlace ? 1 : 0, masks, fillState, incremental ? 1 : 0);
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;
 }

@@ -9,7 +9,7 @@ it can be captured into a HIP graph.
 import numpy as np
 import torch
 
-from .plugin import Plugin, TensorDesc
+from .plugin import OPT_PERSISTENT_INDEX, Plugin, TensorDesc
 from .spconv_index import index_blob
 from .spconv_mm import mm_blob
 
@@ -41,8 +41,9 @@ def densify(x):
 class Rulebook:
     """Outputs of one SPConvIdx enqueue, cached under an indice key."""
 
-    def __init__(self, index, num_index, out_coors, num_act_out, out_grid, in_tensor):
+    def __init__(self, index, num_index, out_coors, num_act_out, out_grid, in_tensor, plugin=None):
         self.index, self.num_index = index, num_index
+        self.plugin = plugin  # the SPConvIdx operator that wrote it: convolutions of the key link to it
         self.out_coors, self.num_act_out, self.out_grid = out_coors, num_act_out, out_grid
         self.in_coors, self.num_act_in, self.in_grid = in_tensor.coors, in_tensor.num_act, in_tensor.grid
 
@@ -59,6 +60,8 @@ class SparseConvLayer:
         self.idx_plugin = Plugin("SPConvIdx%dd" % nd, index_blob(
             spec["ksize"], spec["stride"], spec["padding"], spec["dilation"], (0,) * nd, self.max_num_act_out,
             spec["subm"], spec.get("transpose", False)))
+        # the index tensor is allocated once below and written by this operator only
+        self.idx_plugin.set_option(OPT_PERSISTENT_INDEX, 1)
         self.mm_plugin = Plugin("SPConvMM", mm_blob(
             spec["ksize"], spec["cin"], spec["cout"], self.max_num_act_out, spec["subm"], spec.get("inverse", False),
             weight, bias, relu=spec.get("relu", False), act_scale_in=float(spec.get("s_in", 1.0)),
@@ -82,9 +85,9 @@ class SparseConvLayer:
         self.idx_plugin.enqueue(st["in_descs"], st["out_descs"], [x.coors, x.num_act, None], st["outs"], st["ws"])
         outs = st["outs"]
         if self.spec["subm"]:  # SubM: outputs sit on the input voxels (test_middle_encoder.py:68-69)
-            return Rulebook(outs[0], outs[1], x.coors, x.num_act, x.grid, x)
+            return Rulebook(outs[0], outs[1], x.coors, x.num_act, x.grid, x, self.idx_plugin)
         out_grid = list(st["out_descs"][4].shape()[2:])
-        return Rulebook(outs[0], outs[1], outs[2], outs[3], out_grid, x)
+        return Rulebook(outs[0], outs[1], outs[2], outs[3], out_grid, x, self.idx_plugin)
 
     # -- convolution ------------------------------------------------------------
     def forward(self, x, rulebooks):
@@ -93,15 +96,22 @@ class SparseConvLayer:
         if rb is None:
             rb = rulebooks[key] = self.build_rulebook(x)
         feats = x.feats
-        if self._mm_state is None or self._mm_state["in_rows"] != feats.shape[0]:
-            in_descs = [TensorDesc.of_tensor(t) for t in (feats, rb.num_act_in, rb.num_act_out, rb.index, rb.num_index)]
+        inverse = bool(self.spec.get("inverse", False))
+        # an inverse convolution runs the rulebook backwards: its inputs sit on the rulebook's output sites and its
+        # outputs on the rulebook's input sites (reference: SPConvMM `inverse`, trt/spconv/mm_trt.cu:171-176)
+        num_in, num_out = (rb.num_act_out, rb.num_act_in) if inverse else (rb.num_act_in, rb.num_act_out)
+        if self._mm_state is None or self._mm_state["in_rows"] != feats.shape[0] or self._mm_state["rb"] is not rb.plugin:
+            in_descs = [TensorDesc.of_tensor(t) for t in (feats, num_in, num_out, rb.index, rb.num_index)]
             out_descs = self.mm_plugin.output_descs(in_descs)
+            self.mm_plugin.link_rulebook(rb.plugin)
             self.mm_plugin.configure(in_descs, out_descs)
             out = torch.empty(out_descs[0].shape(), dtype=self.dtype, device=self.device)
-            self._mm_state = dict(in_rows=feats.shape[0], in_descs=in_descs, out_descs=out_descs, out=out)
+            self._mm_state = dict(in_rows=feats.shape[0], in_descs=in_descs, out_descs=out_descs, out=out, rb=rb.plugin)
         st = self._mm_state
-        self.mm_plugin.enqueue(st["in_descs"], st["out_descs"],
-                               [feats, rb.num_act_in, rb.num_act_out, rb.index, rb.num_index], [st["out"]])
+        self.mm_plugin.enqueue(st["in_descs"], st["out_descs"], [feats, num_in, num_out, rb.index, rb.num_index],
+                               [st["out"]])
+        if inverse:
+            return SparseTensor(st["out"], rb.in_coors, rb.num_act_in, rb.in_grid, x.batch)
         return SparseTensor(st["out"], rb.out_coors, rb.num_act_out, rb.out_grid, x.batch)
 
 
@@ -179,16 +189,21 @@ def plan_capacities(layers, n_in, counts=None):
 
     SubM layers keep the capacity of their input.  A strided layer's capacity is
     the measured output count rounded up to 1024 when ``counts[name]`` is given,
-    else the safe bound 8x the input capacity.
+    else the safe bound 8x the input capacity.  An inverse layer outputs on the sites its key's
+    rulebook was built from, so it takes that input's capacity.
     """
     caps = []
     cap_of = {"input": n_in}
+    key_in_cap = {}  # capacity of the input a key's rulebook was built on: what an inverse layer of the key outputs
     cur = n_in
     for spec in layers:
         src = spec.get("src")
         if src is not None:
             cur = cap_of[src.split("+")[0]]
-        if spec["subm"]:
+        key_in_cap.setdefault(spec["key"], cur)
+        if spec.get("inverse", False):
+            cap = key_in_cap[spec["key"]]
+        elif spec["subm"]:
             cap = cur
         elif counts is not None and spec["name"] in counts:
             cap = _round_up(int(counts[spec["name"]]), 1024)

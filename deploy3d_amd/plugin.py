@@ -27,8 +27,9 @@ EXPORTS = [
     "d3d_create", "d3d_clone", "d3d_destroy", "d3d_plugin_type", "d3d_plugin_version", "d3d_serialize_size",
     "d3d_serialize", "d3d_num_outputs", "d3d_output_dims", "d3d_output_dtype", "d3d_supports_format",
     "d3d_configure", "d3d_workspace_size", "d3d_enqueue", "d3d_last_error", "d3d_num_ops", "d3d_op_name",
-    "d3d_clear_cache", "d3d_enqueue_static",
+    "d3d_enqueue_static", "d3d_link_rulebook", "d3d_set_option",
 ]
+OPT_PERSISTENT_INDEX = 1
 
 
 class EngineError(RuntimeError):
@@ -108,7 +109,10 @@ def load_library(path=None):
     lib.d3d_num_ops.restype = i32
     lib.d3d_op_name.restype = ctypes.c_char_p
     lib.d3d_op_name.argtypes = [i32]
-    lib.d3d_clear_cache.restype = None
+    lib.d3d_link_rulebook.restype = i32
+    lib.d3d_link_rulebook.argtypes = [vp, vp]
+    lib.d3d_set_option.restype = i32
+    lib.d3d_set_option.argtypes = [vp, i32, ctypes.c_int64]
     _lib = lib
     return lib
 
@@ -196,6 +200,14 @@ class Plugin:
         return self._lib.d3d_workspace_size(self._h, _desc_array(in_descs), len(in_descs), _desc_array(out_descs),
                                             len(out_descs))
 
+    def link_rulebook(self, idx_plugin):
+        """SPConvMM only: this node's index tensor is the output of ``idx_plugin`` (None removes the link), so the
+        rulebook operator writes the neighbour table and tile masks itself and this node uses them."""
+        _check(self._lib.d3d_link_rulebook(self._h, None if idx_plugin is None else idx_plugin._h))
+
+    def set_option(self, option, value):
+        _check(self._lib.d3d_set_option(self._h, int(option), int(value)))
+
     def enqueue(self, in_descs, out_descs, inputs, outputs, workspace=None, stream=None):
         """inputs / outputs: torch tensors (or None for shape-only tensors); returns the raw status check."""
         def ptrs(ts):
@@ -221,7 +233,3 @@ STATIC_SCRATCH_BYTES = 64 << 20
 
 def torch_dtype(d3d_dtype):
     return _D3D_TO_TORCH[d3d_dtype]
-
-
-def clear_cache():
-    load_library().d3d_clear_cache()

@@ -39,6 +39,13 @@ def _workspace(nbytes, device):
     return ws
 
 
+def index_plugin(kernel_size, stride, padding, dilation, out_padding, max_num_act_out, subm, transpose):
+    """The operator instance ``spconv_index_nd`` runs for these attributes (one per distinct attribute blob); what
+    ``spconv_mm(..., rulebook=...)`` links a convolution to."""
+    blob = index_blob(kernel_size, stride, padding, dilation, out_padding, max_num_act_out, subm, transpose)
+    return _plugin("SPConvIdx%dd" % len(kernel_size), blob)
+
+
 def spconv_index_nd(in_coors, num_act_in, in_spatial_shape, kernel_size, stride, padding, dilation, out_padding,
                     max_num_act_out, subm, transpose):
     """SPConvIdx{N}d for N = len(kernel_size) in 1..4.
@@ -53,8 +60,7 @@ def spconv_index_nd(in_coors, num_act_in, in_spatial_shape, kernel_size, stride,
     if in_coors.dtype != torch.int32 or num_act_in.dtype != torch.int32:
         raise TypeError("coordinates and counts must be int32")
     in_coors = in_coors.contiguous()
-    blob = index_blob(kernel_size, stride, padding, dilation, out_padding, max_num_act_out, subm, transpose)
-    plugin = _plugin("SPConvIdx%dd" % nd, blob)
+    plugin = index_plugin(kernel_size, stride, padding, dilation, out_padding, max_num_act_out, subm, transpose)
     in_descs = [TensorDesc.of_tensor(in_coors), TensorDesc.of_tensor(num_act_in),
                 TensorDesc.of(tuple(in_spatial_shape.shape), torch.int32)]
     out_descs = plugin.output_descs(in_descs)

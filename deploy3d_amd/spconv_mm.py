@@ -51,16 +51,21 @@ def run_mm(plugin, in_feats, num_act_in, num_act_out, index, num_index, out=None
 
 
 def spconv_mm(in_feats, num_act_in, num_act_out, index, num_index, kernel_size, in_channels, out_channels,
-              max_num_act_out, subm, inverse, weight, bias=None, relu=False, act_scale_in=1.0, act_scale_out=1.0):
+              max_num_act_out, subm, inverse, weight, bias=None, relu=False, act_scale_in=1.0, act_scale_out=1.0,
+              rulebook=None):
     """out[maxNumActOut, Cout] = bias + sum over taps of in[gather] @ W[tap] scattered to out rows.
 
     Same positional arguments as the reference's ``spconv_mm``; ``weight`` is the
     flat fp32 [kVol, Cin, Cout] array, ``bias`` fp32 [Cout] or None.  The keyword arguments are this
-    build's extensions: a fused ReLU and, for int8 features, the activation scales of input and output.
+    build's extensions: a fused ReLU; for int8 features, the activation scales of input and output; and
+    ``rulebook``, the SPConvIdx operator instance that wrote ``index`` (``spconv_index.index_plugin``): the
+    convolution is linked to it and reads the neighbour table that operator wrote instead of deriving one from the
+    index tensor (which is what happens without it, and for any tensor that operator did not write last).
     """
     blob = mm_blob(kernel_size, in_channels, out_channels, max_num_act_out, subm, inverse, weight, bias, relu,
                    act_scale_in, act_scale_out)
     plugin = get_plugin(blob)
+    plugin.link_rulebook(rulebook)
     return run_mm(plugin, in_feats.contiguous(), num_act_in, num_act_out, index, num_index)
 
 

@@ -143,7 +143,7 @@ int32_t d3d_enqueue(d3d_plugin* p, const d3d_tensor_desc* in_desc, const d3d_ten
  * BEVDensify and SimpleMeanEncoder with the workspace taken from a fixed array of D3D_STATIC_SCRATCH_BYTES that is
  * part of the library's device image (each GPU the library runs on holds it until the process ends).  Calls no
  * hipMalloc / hipFree; an operator whose d3d_workspace_size() exceeds the array returns D3D_ERR_WORKSPACE, and
- * SPConvMM (which keeps derived tables in library-allocated memory) returns D3D_ERR_UNSUPPORTED.  All calls on one
+ * SPConvMM (which may have to derive a table into library-allocated memory) returns D3D_ERR_UNSUPPORTED.  All calls on one
  * GPU share the array: calls that overlap in time on one GPU (two streams, two threads) race; calls ordered on
  * one stream do not, since every operator clears what it needs zeroed itself. */
 #define D3D_STATIC_SCRATCH_BYTES (64u << 20)
@@ -158,10 +158,30 @@ const char* d3d_last_error(void);
 int32_t d3d_num_ops(void);
 const char* d3d_op_name(int32_t i);
 
-/* Frees every cached neighbour table (the derived, output-major form of an
- * index tensor that convolutions sharing one indice key reuse).  No reference
- * counterpart: the reference keeps no derived state between enqueues. */
-void d3d_clear_cache(void);
+/* No counterpart in the reference, whose SPConvMM re-reads the index tensor on every enqueue
+ * (trt/spconv/mm_trt.cu:166-170) and so does an SPConvMM of this library that nobody linked: it derives the
+ * output-major neighbour table its kernels read from the index tensor it is handed, every time.
+ * d3d_link_rulebook(mm, idx) tells the convolution `mm` that its index tensor (inputs 3 and 4) is output 0 and 1 of
+ * the rulebook operator `idx` - the edge an engine builder sees in the graph.  From then on `idx` writes the
+ * table (and the tap masks of 64-row tiles) itself while it compacts the pairs, into device memory that the two
+ * handles own together (allocated here, freed when the last of them is destroyed), and `mm` uses it whenever the
+ * index tensor it is handed is the one `idx` wrote last, at the same shapes; any other tensor is still derived.
+ * Several convolutions may be linked to one rulebook operator (the reference's indice_key sharing);
+ * idx = NULL removes the link.  What the link cannot see: a caller that edits the index tensor in place between
+ * the two enqueues - do not link such graphs.  A convolution accumulates one input per (tap, output row): an
+ * index tensor that names several (duplicate input coordinates) keeps the highest input row. */
+int32_t d3d_link_rulebook(d3d_plugin* mm, d3d_plugin* idx);
+
+/* Options, none of which the reference has.
+ * D3D_OPT_PERSISTENT_INDEX (SPConvIdx{N}d; value 0 / 1): the caller promises that the index tensor this handle
+ * writes (output 0) is the same buffer on every enqueue and that nothing else writes to it in between - true for
+ * a runner that owns its buffers, not for a buffer an executor recycles for other tensors.  The operator then sets
+ * to -1 only the slots its previous pass used and the new one does not, instead of the whole tensor at capacity
+ * (reference: cudaMemsetAsync of the whole tensor, trt/spconv/index.cu:352-354); after every enqueue the tensor
+ * still reads -1 in every unused slot.  The first enqueue on a buffer, and the first after the buffer or its shape
+ * changed, fill it whole. */
+enum { D3D_OPT_PERSISTENT_INDEX = 1 };
+int32_t d3d_set_option(d3d_plugin* p, int32_t option, int64_t value);
 
 #ifdef __cplusplus
 }

@@ -3,6 +3,10 @@ import sys
 
 import pytest
 
+# the library honours its tuning / test switches (D3D_RULEBOOK, D3D_CONV_STAGED, ...) only in a process that has
+# this set when the library first looks
+os.environ["D3D_DEBUG_ENV"] = "1"
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

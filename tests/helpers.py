@@ -135,10 +135,18 @@ def dense_weight(weight, ksize):
 # GPU wrappers (through the C ABI via deploy3d_amd)
 # ---------------------------------------------------------------------------
 def gpu_rulebook(coords, num_act_in, grid, batch, ksize, stride, padding, dilation, max_num_act_out, subm,
-                 transpose=False, out_padding=None, cap=None):
+                 transpose=False, out_padding=None, cap=None, link=False):
+    """link=True: a placeholder convolution is linked to the operator first, so that this enqueue also writes the
+    neighbour table and tile masks (res["plugin"] is what spconv_mm(..., rulebook=) takes)."""
     import torch
     from deploy3d_amd import spconv_index_nd
+    from deploy3d_amd.spconv_index import index_plugin
+    from deploy3d_amd.spconv_mm import get_plugin, mm_blob
     nd = len(ksize)
+    plugin = index_plugin(ksize, stride, padding, dilation, out_padding or (0,) * nd, max_num_act_out, subm, transpose)
+    if link:
+        get_plugin(mm_blob(ksize, 1, 1, max_num_act_out, subm, False,
+                           np.zeros(int(np.prod(ksize)), np.float32))).link_rulebook(plugin)
     cap = cap or len(coords)
     c = torch.zeros((cap, nd + 1), dtype=torch.int32, device="cuda")
     c[:len(coords)] = torch.from_numpy(np.ascontiguousarray(coords)).cuda()
@@ -147,7 +155,8 @@ def gpu_rulebook(coords, num_act_in, grid, batch, ksize, stride, padding, dilati
     out = spconv_index_nd(c, num, shape, ksize, stride, padding, dilation, out_padding or (0,) * nd, max_num_act_out,
                           subm, transpose)
     torch.cuda.synchronize()
-    res = dict(index=out[0].cpu().numpy(), num_index=int(out[1].item()), dev=out, in_coors=c, num_act_in=num)
+    res = dict(index=out[0].cpu().numpy(), num_index=int(out[1].item()), dev=out, in_coors=c, num_act_in=num,
+               plugin=plugin)
     if not subm:
         res.update(out_coors=out[2].cpu().numpy(), num_act_out=int(out[3].item()),
                    out_grid=list(out[4].shape[2:]))

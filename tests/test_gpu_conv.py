@@ -33,7 +33,9 @@ def check_close(got, ref, dtype):
 
 
 def run_case(n, grid, ksize, stride, padding, cin, cout, dtype, subm, with_bias=True, relu=False, inverse=False,
-             seed=0, cap_extra=0):
+             seed=0, cap_extra=0, link=True):
+    """link: the convolution is linked to the rulebook operator and reads the table that operator wrote (an inverse
+    convolution never does); otherwise it derives the table from the index tensor, as an unlinked node does."""
     from deploy3d_amd import spconv_mm
     rng = np.random.default_rng(seed + n + cin * 7 + cout)
     coords = random_cloud(rng, n, grid, 1)
@@ -41,7 +43,7 @@ def run_case(n, grid, ksize, stride, padding, cin, cout, dtype, subm, with_bias=
     kvol = int(np.prod(ksize))
     dil = (1,) * len(ksize)
     max_out = n if subm else n * 8
-    rb = gpu_rulebook(coords, n, grid, 1, ksize, stride, padding, dil, max_out, subm, cap=n + cap_extra)
+    rb = gpu_rulebook(coords, n, grid, 1, ksize, stride, padding, dil, max_out, subm, cap=n + cap_extra, link=link)
     n_out = n if subm else rb["num_act_out"]
     in_rows, out_rows = (n + cap_extra, max_out) if not inverse else (max_out, n + cap_extra)
     feats = round_to(rng.standard_normal((in_rows, cin)), dtype)
@@ -59,7 +61,7 @@ def run_case(n, grid, ksize, stride, padding, cin, cout, dtype, subm, with_bias=
         num_in, num_out = num_out, num_in
     x = torch.from_numpy(feats).to(device="cuda", dtype=TORCH_DTYPE[dtype])
     y = spconv_mm(x, num_in, num_out, idx_dev, num_index_dev, ksize, cin, cout, out_rows, subm, inverse, w, b,
-                  relu=relu)
+                  relu=relu, rulebook=rb["plugin"] if link else None)
     torch.cuda.synchronize()
     got = y.float().cpu().numpy()
     live = n if (subm or inverse) else n_out
@@ -104,22 +106,95 @@ def test_kernel_shapes(engine, ksize, padding):
 
 def test_mirrored_neighbour_table(engine, monkeypatch):
     """SubM with 'same' padding: the compaction writes the output-major table from the mirrored twin of every pair
-    instead of scattering; D3D_RULEBOOK_MIRROR=0 selects the scatter.  Both must give the same features bit for bit,
-    for shuffled rows and for rows in rank order; a SubM geometry without the symmetry (padding (1, 1, 0)) takes the
-    scatter by itself and must still match the oracle."""
-    from deploy3d_amd.plugin import clear_cache
+    instead of scattering; D3D_RULEBOOK_MIRROR=0 selects the scatter, and an unlinked convolution derives the table
+    from the index tensor.  All three must give the same features bit for bit, for shuffled rows and for rows in
+    rank order; a SubM geometry without the symmetry (padding (1, 1, 0)) takes the scatter by itself and must still
+    match the oracle."""
     for ksize, padding in (((3, 3, 3), (1, 1, 1)), ((3, 1, 3), (1, 0, 1)), ((5, 5, 5), (2, 2, 2))):
         monkeypatch.delenv("D3D_RULEBOOK_MIRROR", raising=False)
-        clear_cache()
         a, _ = run_case(3000, (10, 36, 30), ksize, (1, 1, 1), padding, 32, 64, "float16", True, seed=5)
         monkeypatch.setenv("D3D_RULEBOOK_MIRROR", "0")
-        clear_cache()
         b, _ = run_case(3000, (10, 36, 30), ksize, (1, 1, 1), padding, 32, 64, "float16", True, seed=5)
-        assert np.array_equal(a, b)
+        c, _ = run_case(3000, (10, 36, 30), ksize, (1, 1, 1), padding, 32, 64, "float16", True, seed=5, link=False)
+        assert np.array_equal(a, b) and np.array_equal(a, c)
     monkeypatch.delenv("D3D_RULEBOOK_MIRROR", raising=False)
-    clear_cache()
     run_case(3000, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 0), 32, 64, "float16", True, seed=6)
     run_case(3000, (10, 36, 30), (3, 3, 2), (1, 1, 1), (1, 1, 0), 16, 32, "float16", True, seed=7)
+
+
+@pytest.mark.parametrize("subm,stride", [(True, (1, 1, 1)), (False, (2, 2, 2))])
+@pytest.mark.parametrize("cin,cout,dtype", [(64, 64, "float16"), (16, 32, "float16"), (5, 16, "float32")])
+def test_unlinked_convolution_derives_its_table(engine, subm, stride, cin, cout, dtype):
+    """A node nobody linked works from the index tensor alone, like the reference's (trt/spconv/mm_trt.cu:166-170)."""
+    a, _ = run_case(3000, (10, 36, 30), (3, 3, 3), stride, (1, 1, 1), cin, cout, dtype, subm, link=False, seed=11)
+    b, _ = run_case(3000, (10, 36, 30), (3, 3, 3), stride, (1, 1, 1), cin, cout, dtype, subm, link=True, seed=11)
+    assert np.array_equal(a, b)
+
+
+def _mm_on_index(index_np, num_index, n, cin, cout, feats, w, rulebook=None, index_dev=None):
+    from deploy3d_amd import spconv_mm
+    one = torch.tensor([n], dtype=torch.int32, device="cuda")
+    idx = index_dev if index_dev is not None else torch.from_numpy(index_np).cuda()
+    ni = torch.tensor([num_index], dtype=torch.int32, device="cuda")
+    y = spconv_mm(torch.from_numpy(feats).cuda().half(), one, one, idx, ni, (3, 3, 3), cin, cout, n, True, False, w,
+                  rulebook=rulebook)
+    torch.cuda.synchronize()
+    return y.float().cpu().numpy()
+
+
+def test_foreign_and_edited_index_tensors(engine):
+    """The index tensor is the contract: (a) a tensor uploaded from the CPU oracle, which this library never wrote;
+    (b) a library-written tensor overwritten in place with another rulebook, fed to an unlinked node; (c) a linked
+    node handed a tensor at another address than the one its rulebook operator wrote.  Each must give the result
+    of the pairs the tensor holds."""
+    rng = np.random.default_rng(42)
+    grid, n, cin, cout = (10, 36, 30), 2000, 32, 32
+    coords_a = random_cloud(rng, n, grid, 1)
+    coords_b = random_cloud(rng, n, grid, 1)
+    feats = round_to(rng.standard_normal((n, cin)), "float16")
+    w = round_to(rng.standard_normal((27, cin, cout)) / np.sqrt(27 * cin), "float16")
+    geom = ((3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1))
+    ref = {}
+    for name, c in (("a", coords_a), ("b", coords_b)):
+        r = oracle.rulebook(c, n, (1,) + grid, *geom, n, True)
+        ref[name] = (r["index"], r["num_index"], oracle.conv(feats, w, None, r["index"], r["num_index"], n, acc="f64"))
+    # (a) oracle-written tensor
+    got = _mm_on_index(ref["a"][0], ref["a"][1], n, cin, cout, feats, w)
+    check_close(got, ref["a"][2], "float16")
+    # (b) library-written, then edited in place
+    rb = gpu_rulebook(coords_a, n, grid, 1, *geom, n, True, link=True)
+    got = _mm_on_index(None, rb["num_index"], n, cin, cout, feats, w, rulebook=rb["plugin"], index_dev=rb["dev"][0])
+    check_close(got, ref["a"][2], "float16")
+    rb["dev"][0].copy_(torch.from_numpy(ref["b"][0]).cuda())
+    got = _mm_on_index(None, ref["b"][1], n, cin, cout, feats, w, index_dev=rb["dev"][0])
+    check_close(got, ref["b"][2], "float16")
+    # (c) linked node, tensor at another address
+    other = torch.from_numpy(ref["b"][0]).cuda()
+    got = _mm_on_index(None, ref["b"][1], n, cin, cout, feats, w, rulebook=rb["plugin"], index_dev=other)
+    check_close(got, ref["b"][2], "float16")
+
+
+def test_duplicate_pairs_keep_the_highest_input(engine):
+    """An index tensor that names two inputs for one (tap, output) - what duplicate input coordinates produce - is
+    outside what the output-stationary convolution accumulates: it keeps one input per (tap, output), the highest
+    row, on every run (the reference adds both; parity unpinned by the reference's tests, which never feed
+    duplicates)."""
+    n, cin, cout = 256, 32, 32
+    rng = np.random.default_rng(3)
+    feats = round_to(rng.standard_normal((n, cin)), "float16")
+    w = round_to(rng.standard_normal((27, cin, cout)) / np.sqrt(27 * cin), "float16")
+    row_len = 27 * (n + 128)
+    index = np.full((3, row_len), -1, np.int32)
+    # tap 13 (the centre): inputs 5 and 9 both feed output 5; input 7 feeds output 7
+    index[0, :3] = (5, 7, 9)
+    index[1, :3] = (5, 7, 5)
+    index[2, :3] = 13
+    keep = index.copy()
+    keep[:, 0] = -1  # the pair (5 -> 5) loses against (9 -> 5)
+    ref = oracle.conv(feats, w, None, keep, 128, n, acc="f64")
+    for _ in range(3):
+        got = _mm_on_index(index, 128, n, cin, cout, feats, w)
+        check_close(got, ref, "float16")
 
 
 @pytest.mark.parametrize("tile_rows", [128, 256, 512])

@@ -172,6 +172,71 @@ def test_single_voxel_and_full_block(engine):
     assert live.sum() == expected
 
 
+def test_persistent_index_tensor(engine):
+    """D3D_OPT_PERSISTENT_INDEX: one handle, one index tensor, passes of different sizes.  After every enqueue the
+    whole tensor equals the oracle's (every unused slot -1) although only the first pass fills it at capacity.
+    The documented limit of the promise: a value the caller writes past the used part is not the library's to
+    clean (it is wiped without the option)."""
+    import torch
+    from deploy3d_amd.plugin import OPT_PERSISTENT_INDEX, Plugin, TensorDesc
+    from deploy3d_amd.spconv_index import index_blob
+    from deploy3d_amd.spconv_mm import get_plugin, mm_blob
+    grid, cap = (12, 40, 33), 4000
+    rng = np.random.default_rng(77)
+    for subm, stride, with_table in ((True, (1, 1, 1), True), (False, (2, 2, 2), True), (True, (1, 1, 1), False)):
+        max_out = cap if subm else 8 * cap
+        args = ((3, 3, 3), stride, (1, 1, 1), (1, 1, 1))
+        plugin = Plugin("SPConvIdx3d", index_blob(*args, (0, 0, 0), max_out, subm, False))
+        plugin.set_option(OPT_PERSISTENT_INDEX, 1)
+        if with_table:
+            get_plugin(mm_blob((3, 3, 3), 1, 1, max_out, subm, False, np.zeros(27, np.float32))).link_rulebook(plugin)
+        coors = torch.zeros((cap, 4), dtype=torch.int32, device="cuda")
+        num = torch.zeros(1, dtype=torch.int32, device="cuda")
+        in_descs = [TensorDesc.of_tensor(coors), TensorDesc.of_tensor(num), TensorDesc.of((1, 0) + grid, torch.int32)]
+        out_descs = plugin.output_descs(in_descs)
+        outs = [torch.empty(d.shape(), dtype=torch.int32, device="cuda") for d in out_descs]
+        outs[0].fill_(12345)  # the first pass must not rely on what the buffer held
+        ws = torch.empty(max(1, plugin.workspace_size(in_descs, out_descs)), dtype=torch.uint8, device="cuda")
+        out_grid = (1,) + (grid if subm else tuple(out_descs[4].shape()[2:]))
+        for n in (3000, 500, 0, 4000, 1200):
+            coords = random_cloud(rng, n, grid, 1) if n else np.zeros((0, 4), np.int32)
+            coors.zero_()
+            coors[:n] = torch.from_numpy(coords).cuda()
+            num.fill_(n)
+            plugin.enqueue(in_descs, out_descs, [coors, num, None], outs, ws)
+            torch.cuda.synchronize()
+            ref = oracle.rulebook(coors.cpu().numpy(), n, out_grid, *args, max_out, subm)
+            index = outs[0].cpu().numpy()
+            ni = int(outs[1].item())
+            assert ni == ref["num_index"]
+            if subm:
+                np.testing.assert_array_equal(index, ref["index"])
+            else:
+                assert (index[:, ni:] == -1).all()
+                c_ref, t_ref = oracle.canonical(ref["index"], ref["num_index"], ref["out_coors"], ref["num_act_out"])
+                c_got, t_got = oracle.canonical(index, ni, outs[2].cpu().numpy(), int(outs[3].item()))
+                np.testing.assert_array_equal(c_got, c_ref)
+                np.testing.assert_array_equal(t_got, t_ref)
+            check_index_structure(index, ni, 27, cap)
+        # a caller's write past the used part survives the next pass of a persistent tensor ...
+        outs[0][1, -1] = 777
+        plugin.enqueue(in_descs, out_descs, [coors, num, None], outs, ws)
+        torch.cuda.synchronize()
+        assert int(outs[0][1, -1].item()) == 777
+        # ... and not that of an ordinary one
+        plugin.set_option(OPT_PERSISTENT_INDEX, 0)
+        plugin.enqueue(in_descs, out_descs, [coors, num, None], outs, ws)
+        torch.cuda.synchronize()
+        assert int(outs[0][1, -1].item()) == -1
+        # switching the option on again starts with a full fill
+        plugin.set_option(OPT_PERSISTENT_INDEX, 1)
+        outs[0][2, -2] = 778
+        plugin.enqueue(in_descs, out_descs, [coors, num, None], outs, ws)
+        torch.cuda.synchronize()
+        assert int(outs[0][2, -2].item()) == -1
+        plugin.close()
+
+
 def _random_geometry(rng):
     """A random but valid layer: 1 to 4 dims, kernel 1..5, stride 1..3, padding 0..2, dilation 1..2."""
     nd = int(rng.integers(1, 5))
