@@ -406,12 +406,30 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
 
 // Configuration per layer shape, measured on the layers of a VoxelNet backbone (120k voxels): rows per wavefront
 // 16 * MT, wavefronts per workgroup.  64 x 64 and narrower tiles afford 8 wavefronts; 128 output channels double
-// the accumulators, so the wavefront tile halves.
+// the accumulators, so the wavefront tile halves.  Layers with few rows (the 128-channel stages: 47 000 rows are
+// 186 tiles of 256 rows for 256 CUs) pick the workgroup size whose tile count loads the CUs most evenly: the
+// time of a layer that fits one round is that of ONE tile, so 248 tiles of 192 rows beat 186 of 256.
 template <class T, int CIN, int COUT>
 int32_t launchPipeShape(const ConvArgs& a, hipStream_t stream) {
-  if constexpr (CIN == 64 && COUT == 64) return launchPipeCfg<T, CIN, COUT, 4, 8>(a, stream);
-  else if constexpr (COUT >= 128) return launchPipeCfg<T, CIN, COUT, 2, 8>(a, stream);
-  else return launchPipeCfg<T, CIN, COUT, 4, 4>(a, stream);
+  if constexpr (CIN == 64 && COUT == 64) {
+    return launchPipeCfg<T, CIN, COUT, 4, 8>(a, stream);
+  } else if constexpr (COUT >= 128) {
+    int best = 8;
+    int64_t bestCost = 0;
+    for (int waves = 8; waves >= 4; waves -= 2) {
+      const int64_t tm = 32 * waves, tiles = (a.outRows + tm - 1) / tm;
+      const int64_t cost = (tiles + 255) / 256 * tm;  // rows the busiest CU multiplies
+      if (waves == 8 || cost < bestCost) {
+        best = waves;
+        bestCost = cost;
+      }
+    }
+    if (best == 6) return launchPipeCfg<T, CIN, COUT, 2, 6>(a, stream);
+    if (best == 4) return launchPipeCfg<T, CIN, COUT, 2, 4>(a, stream);
+    return launchPipeCfg<T, CIN, COUT, 2, 8>(a, stream);
+  } else {
+    return launchPipeCfg<T, CIN, COUT, 4, 4>(a, stream);
+  }
 }
 
 template <class T>

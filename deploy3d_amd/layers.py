@@ -146,6 +146,7 @@ class SparseBackbone:
             for st in side.values():
                 st.wait_event(fork)
         rulebooks = {}
+        inputs = {}
         pending = {}
         strided_coords = {}  # coordinate tensor written by a strided rulebook -> main-stream event after its wait
         outs = {"input": x}
@@ -159,6 +160,7 @@ class SparseBackbone:
                 inp = SparseTensor(a.feats + b.feats, a.coors, a.num_act, a.grid, a.batch)
             else:
                 inp = outs[src]
+            inputs[spec["name"]] = inp
             key = spec["key"]
             if side is not None and key not in rulebooks:
                 subm = bool(spec["subm"])
@@ -180,6 +182,7 @@ class SparseBackbone:
             cur = lyr.forward(inp, rulebooks)
             outs[spec["name"]] = cur
         self.rulebooks = rulebooks
+        self.inputs = inputs    # layer name -> the SparseTensor it read
         self.outputs = outs
         return cur
 
