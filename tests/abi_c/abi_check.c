@@ -26,6 +26,8 @@ typedef const char* (*str_fn)(void);
 typedef const char* (*type_fn)(const d3d_plugin*);
 typedef int32_t (*count_fn)(void);
 typedef const char* (*name_fn)(int32_t);
+typedef int32_t (*link_fn)(d3d_plugin*, d3d_plugin*);
+typedef int32_t (*option_fn)(d3d_plugin*, int32_t, int64_t);
 
 int main(int argc, char** argv) {
   CHECK(argc == 2);
@@ -45,8 +47,10 @@ int main(int argc, char** argv) {
   type_fn plugin_type = (type_fn)dlsym(lib, "d3d_plugin_type");
   count_fn num_ops = (count_fn)dlsym(lib, "d3d_num_ops");
   name_fn op_name = (name_fn)dlsym(lib, "d3d_op_name");
+  link_fn link_rulebook = (link_fn)dlsym(lib, "d3d_link_rulebook");
+  option_fn set_option = (option_fn)dlsym(lib, "d3d_set_option");
   CHECK(create && clone && destroy && ser_size && serialize && num_outputs && output_dims && last_error &&
-        plugin_type && num_ops && op_name);
+        plugin_type && num_ops && op_name && link_rulebook && set_option);
 
   CHECK(num_ops() >= 5);
   CHECK(strcmp(op_name(2), "SPConvIdx3d") == 0);
@@ -78,6 +82,25 @@ int main(int argc, char** argv) {
 
   d3d_plugin* q = NULL;
   CHECK(clone(p, &q) == D3D_OK && q && ser_size(q) == sizeof(blob));
+
+  /* SPConvMMPluginParam: 4 x int32, 3 x u8, then fp32 W[kVol*Cin*Cout] (1x1x1 kernel, 2 -> 2 channels) */
+  unsigned char mm_blob[19 + 16];
+  const int32_t mm_fields[4] = {1, 2, 2, 5000};
+  const float mm_w[4] = {1.f, 0.f, 0.f, 1.f};
+  memcpy(mm_blob, mm_fields, 16);
+  mm_blob[16] = 0; mm_blob[17] = 0; mm_blob[18] = 0;
+  memcpy(mm_blob + 19, mm_w, 16);
+  d3d_plugin* mm = NULL;
+  CHECK(create("SPConvMM", "2.0", mm_blob, sizeof(mm_blob), &mm) == D3D_OK && mm);
+  /* linking checks its operands before it touches the device */
+  CHECK(link_rulebook(p, q) == D3D_ERR_BAD_ARG);           /* first handle is not a convolution */
+  CHECK(link_rulebook(mm, mm) == D3D_ERR_BAD_ARG);         /* second handle is not a rulebook operator */
+  CHECK(link_rulebook(mm, p) == D3D_ERR_BAD_ARG);          /* kernel volume 1 against 27 */
+  CHECK(link_rulebook(mm, NULL) == D3D_OK);                /* removing a link that is not there */
+  CHECK(set_option(mm, D3D_OPT_PERSISTENT_INDEX, 1) == D3D_ERR_UNSUPPORTED && strlen(last_error()) > 0);
+  CHECK(set_option(p, 12345, 1) == D3D_ERR_UNSUPPORTED);
+  CHECK(set_option(NULL, D3D_OPT_PERSISTENT_INDEX, 1) == D3D_ERR_BAD_ARG);
+  destroy(mm);
   destroy(q);
   destroy(p);
 
