@@ -53,6 +53,7 @@ struct RbGeom {
   int p[kMaxSpatial];
   int d[kMaxSpatial];
   int shape[kMaxSpatial + 1];   // output grid: batch, then 4 spatial extents
+  int inShape[kMaxSpatial + 1]; // input grid, same layout: a live row outside it takes part in no pair
   int kVol;
   int transpose;
 };
@@ -115,6 +116,8 @@ struct ConvArgs {
   int64_t inRows;         // capacity rows of inFeats
   int64_t outRows;        // maxNumActOut
   const void* in;
+  const void* inNarrow;   // the rows as the caller passed them, cinNarrow channels wide (in may be a widened copy)
+  int cinNarrow;
   void* out;
   const float* weightsF32;  // device fp32 [kVol, cin, cout], values already rounded to the storage type
   const void* weightsMfma;  // device storage-type, MFMA fragment-major (see MMPlugin::configure) or null

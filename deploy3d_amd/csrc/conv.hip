@@ -260,6 +260,14 @@ int32_t launchConv(const ConvArgs& a, hipStream_t stream) {
     if (a.pipe >= 0 && a.staged == 0 && a.tileRows == 0)
       rc = a.dtype == D3D_HALF ? launchPipeHalf(a, stream) : launchPipeBf16(a, stream);
     if (rc == D3D_ERR_UNSUPPORTED) rc = a.dtype == D3D_HALF ? launchMfmaHalf(a, stream) : launchMfmaBf16(a, stream);
+    if (rc == D3D_ERR_UNSUPPORTED && a.weightsF32 && a.inNarrow) {
+      // no MFMA instantiation fits (a kernel volume whose index rows exceed LDS, 7x7x7 at 128 channels say): the
+      // narrow kernel takes any kernel volume (the reference accepts any, trt/spconv/mm.h:35-71)
+      ConvArgs b = a;
+      b.in = a.inNarrow;
+      b.cin = a.cinNarrow;
+      rc = a.dtype == D3D_HALF ? launchNarrow<_Float16>(b, stream) : launchNarrow<__bf16>(b, stream);
+    }
   } else {
     switch (a.dtype) {
       case D3D_FLOAT: rc = launchNarrow<float>(a, stream); break;

@@ -361,8 +361,9 @@ struct IdxPlugin final : d3d_plugin {
   }
   int32_t configure(const d3d_tensor_desc*, int32_t, const d3d_tensor_desc*, int32_t) override { return D3D_OK; }
 
-  RbGeom geometry(const int32_t* outGrid /* [B, spatial...] */) const {
+  RbGeom geometry(const int32_t* outGrid /* [B, spatial...] */, const int32_t* inGrid = nullptr) const {
     RbGeom g{};
+    if (!inGrid) inGrid = outGrid;
     g.nd = nd;
     const int pad = kMaxSpatial - nd;
     for (int i = 0; i < kMaxSpatial; ++i) {
@@ -372,8 +373,10 @@ struct IdxPlugin final : d3d_plugin {
       g.p[i] = real ? padding[i - pad] : 0;
       g.d[i] = real ? dilation[i - pad] : 1;
       g.shape[i + 1] = real ? outGrid[1 + i - pad] : 1;
+      g.inShape[i + 1] = real ? inGrid[1 + i - pad] : 1;
     }
     g.shape[0] = outGrid[0];
+    g.inShape[0] = inGrid[0];
     g.kVol = kVol();
     g.transpose = transpose ? 1 : 0;
     return g;
@@ -423,7 +426,10 @@ struct IdxPlugin final : d3d_plugin {
         return D3D_ERR_BAD_ARG;
       }
     }
-    const RbGeom g = geometry(grid);
+    int32_t inGrid[kMaxSpatial + 1];
+    inGrid[0] = inDesc[2].dims[0];
+    for (int i = 0; i < nd; ++i) inGrid[1 + i] = inDesc[2].dims[2 + i];
+    const RbGeom g = geometry(grid, inGrid);
     std::lock_guard<std::mutex> lock(link->mutex);
     RbSide side{};
     const size_t tableBytes = static_cast<size_t>(kVol()) * static_cast<size_t>(maxNumActOut) * sizeof(int32_t);
@@ -811,6 +817,8 @@ struct MMPlugin final : d3d_plugin {
     a.inRows = inDesc[0].dims[0];
     a.outRows = outRows;
     a.in = inputs[0];
+    a.inNarrow = inputs[0];
+    a.cinNarrow = cin;
     if (dev->cinMfma > cin && (dtype == D3D_INT8 || ((reinterpret_cast<uintptr_t>(outputs[0]) & 15) == 0 &&
                                                      debugEnv("D3D_CONV_NO_PAD") == nullptr))) {  // narrow layer: widen the rows, then MFMA
       if (!widened) widened = std::make_shared<DeviceBuffer>();

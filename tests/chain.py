@@ -46,14 +46,17 @@ def oracle_chain(cfg, threads=1, acc="f64"):
                 rb["out_grid"] = og
             rb["pairs"] = int((rb["index"][2, :rb["num_index"]] >= 0).sum())
             rb["in_coors"] = x["coords"]
+            rb["in_grid"] = x["grid"]
             rulebooks[spec["key"]] = rb
-        n_out = rb["num_act_out"]
+        # an inverse layer runs its key's rulebook backwards: outputs on the sites the rulebook was built from
+        inverse = bool(spec.get("inverse", False))
+        n_out = len(rb["in_coors"]) if inverse else rb["num_act_out"]
         y = oracle.conv(x["feats"], round_to(w, dtype), round_to(b, dtype), rb["index"], rb["num_index"], n_out,
-                        acc=acc, threads=threads)
+                        inverse=inverse, acc=acc, threads=threads)
         if spec.get("relu"):
             y = np.maximum(y, 0)
-        cur = dict(feats=round_to(y, dtype), exact=y, coords=rb["out_coors"], grid=rb["out_grid"],
-                   pairs=rb["pairs"], key=spec["key"])
+        cur = dict(feats=round_to(y, dtype), exact=y, coords=rb["in_coors"] if inverse else rb["out_coors"],
+                   grid=rb["in_grid"] if inverse else rb["out_grid"], pairs=rb["pairs"], key=spec["key"])
         outs[spec["name"]] = cur
     outs["_rulebooks"] = rulebooks
     return outs

@@ -44,6 +44,33 @@ def compare_chain(cfg, net, ref, tol_scale=1.0):
             assert err <= 2e-2 * rms * tol_scale, (spec["name"], err, rms)
 
 
+def test_down_up_chain_with_inverse_convolution(engine):
+    """An encoder-decoder wiring through the layer runner: strided down (key d), SubM at the lower resolution, then
+    the inverse convolution of key d back onto the input sites, then a SubM that shares the first layer's key.  The
+    inverse layer's outputs carry the coordinates, live count, grid and capacity of the rulebook's INPUT side
+    (reference: SPConvMM `inverse`, trt/spconv/mm_trt.cu:171-176); every layer against the oracle chain."""
+    from deploy3d_amd import synth
+    grid, n = (16, 96, 96), 5000
+    coords = synth.coords_lidar(synth.seed(0, 0), grid, n)
+    n = len(coords)
+    feats = synth.normal(synth.seed(0, 1), (n, 16))
+    specs = [
+        synth.layer("s0", "subm0", True, (3, 3, 3), 16, 16, padding=(1, 1, 1)),
+        synth.layer("down", "d", False, (3, 3, 3), 16, 32, stride=(2, 2, 2), padding=(1, 1, 1)),
+        synth.layer("mid", "subm1", True, (3, 3, 3), 32, 32, padding=(1, 1, 1)),
+        dict(synth.layer("up", "d", False, (3, 3, 3), 32, 16, stride=(2, 2, 2), padding=(1, 1, 1)), inverse=True),
+        synth.layer("s1", "subm0", True, (3, 3, 3), 16, 16, padding=(1, 1, 1)),
+    ]
+    cfg = dict(coords=coords, feats=feats, grid=grid, dtype="float16", layers=specs,
+               weights=[synth.layer_weights(0, i, s) for i, s in enumerate(specs)])
+    ref = chain.oracle_chain(cfg)
+    net, x, y = run_gpu_chain(cfg, counts={"down": len(ref["down"]["coords"])})
+    compare_chain(cfg, net, ref)
+    up = net.outputs["up"]
+    assert up.grid == list(grid) and up.coors.data_ptr() == x.coors.data_ptr() and up.feats.shape == (n, 16)
+    assert int(y.num_act.item()) == n
+
+
 def compare_rulebooks(cfg, net, ref):
     """Every rulebook of the pass against the oracle's, bit for bit in canonical form: output coordinates sorted,
     gather and scatter ids relabelled by the rank of their coordinate, triples (tap, gather, scatter) sorted."""

@@ -104,6 +104,13 @@ def test_kernel_shapes(engine, ksize, padding):
     run_case(2500, (10, 36, 30), ksize, (1, 1, 1), padding, 32, 64, "float16", True)
 
 
+def test_large_kernel_volume_falls_back(engine):
+    """7x7x7 at 128 channels fits no MFMA instantiation (343 taps of index rows and weights exceed LDS): the narrow
+    kernel takes over instead of an error status; the reference accepts any kernel volume."""
+    run_case(400, (12, 16, 16), (7, 7, 7), (1, 1, 1), (3, 3, 3), 128, 128, "float16", True, seed=31)
+    run_case(400, (12, 16, 16), (7, 7, 7), (1, 1, 1), (3, 3, 3), 16, 128, "bfloat16", True, seed=32, link=False)
+
+
 def test_mirrored_neighbour_table(engine, monkeypatch):
     """SubM with 'same' padding: the compaction writes the output-major table from the mirrored twin of every pair
     instead of scattering; D3D_RULEBOOK_MIRROR=0 selects the scatter, and an unlinked convolution derives the table
@@ -129,6 +136,50 @@ def test_unlinked_convolution_derives_its_table(engine, subm, stride, cin, cout,
     a, _ = run_case(3000, (10, 36, 30), (3, 3, 3), stride, (1, 1, 1), cin, cout, dtype, subm, link=False, seed=11)
     b, _ = run_case(3000, (10, 36, 30), (3, 3, 3), stride, (1, 1, 1), cin, cout, dtype, subm, link=True, seed=11)
     assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("structure,near", [("blockmap", "1"), ("blockmap", "0"), ("hash", "1")])
+def test_rows_outside_the_grid(engine, monkeypatch, structure, near):
+    """Live rows whose coordinate lies outside the grid are out of contract in the reference (its hash keys alias
+    into other cells, trt/spconv/index.cu:174-182); this engine ignores them: they take part in no pair.  The
+    mirrored table a linked convolution reads and the table an unlinked one derives from the index tensor agree
+    on that, in-grid rows get what the oracle gives for the in-grid cloud alone, and the ignored rows hold the
+    bias."""
+    from deploy3d_amd import spconv_mm
+    monkeypatch.setenv("D3D_RULEBOOK", structure)
+    monkeypatch.setenv("D3D_RULEBOOK_NEAR", near)
+    rng = np.random.default_rng(21)
+    grid, cin, cout = (10, 36, 30), 32, 64
+    inside = random_cloud(rng, 2500, grid, 1)
+    n_in = len(inside)
+    bad = np.array([[0, -1, 5, 5], [0, 3, 36, 2], [0, 3, 4, 30], [1, 2, 2, 2], [0, 10, 0, 0], [-1, 1, 1, 1]], np.int32)
+    where = np.sort(rng.choice(n_in + len(bad), size=len(bad), replace=False))
+    coords = np.zeros((n_in + len(bad), 4), np.int32)
+    is_bad = np.zeros(len(coords), bool)
+    is_bad[where] = True
+    coords[is_bad] = bad
+    coords[~is_bad] = inside
+    n = len(coords)
+    feats = round_to(rng.standard_normal((n, cin)), "float16")
+    w = round_to(rng.standard_normal((27, cin, cout)) / np.sqrt(27 * cin), "float16")
+    b = round_to(rng.standard_normal(cout), "float16")
+    geom = ((3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1))
+    ref_rb = oracle.rulebook(inside, n_in, (1,) + grid, *geom, n_in, True)
+    ref = oracle.conv(feats[~is_bad], w, b, ref_rb["index"], ref_rb["num_index"], n_in, acc="f64")
+    got = {}
+    for link in (True, False):
+        rb = gpu_rulebook(coords, n, grid, 1, *geom, n, True, link=link)
+        x = torch.from_numpy(feats).cuda().half()
+        y = spconv_mm(x, rb["num_act_in"], rb["num_act_in"], rb["dev"][0], rb["dev"][1], (3, 3, 3), cin, cout, n,
+                      True, False, w, b, rulebook=rb["plugin"] if link else None)
+        torch.cuda.synchronize()
+        got[link] = y.float().cpu().numpy()
+        g, s, t = rb["index"][:, :rb["num_index"]]
+        live = t >= 0
+        assert not is_bad[g[live]].any() and not is_bad[s[live]].any()
+    assert np.array_equal(got[True], got[False])
+    check_close(got[True][~is_bad], ref, "float16")
+    np.testing.assert_array_equal(got[True][is_bad], np.broadcast_to(b, (len(bad), cout)))
 
 
 def _mm_on_index(index_np, num_index, n, cin, cout, feats, w, rulebook=None, index_dev=None):

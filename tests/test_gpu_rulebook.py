@@ -172,6 +172,17 @@ def test_single_voxel_and_full_block(engine):
     assert live.sum() == expected
 
 
+def test_ordered_scan_variant(engine, monkeypatch):
+    """D3D_RULEBOOK_ORDERED_SCAN=1 selects acquire-release tickets in the scan pass of the block map: same results."""
+    monkeypatch.setenv("D3D_RULEBOOK_ORDERED_SCAN", "1")
+    test_subm_matches_oracle_bit_exact(engine, SUBM_CASES[9])
+    coords, out_grid, ref, got, kvol = _conv_case(CONV_CASES[1])
+    c_ref, t_ref = oracle.canonical(ref["index"], ref["num_index"], ref["out_coors"], ref["num_act_out"])
+    c_got, t_got = oracle.canonical(got["index"], got["num_index"], got["out_coors"], got["num_act_out"])
+    np.testing.assert_array_equal(c_got, c_ref)
+    np.testing.assert_array_equal(t_got, t_ref)
+
+
 def test_persistent_index_tensor(engine):
     """D3D_OPT_PERSISTENT_INDEX: one handle, one index tensor, passes of different sizes.  After every enqueue the
     whole tensor equals the oracle's (every unused slot -1) although only the first pass fills it at capacity.
