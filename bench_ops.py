@@ -1,7 +1,7 @@
 """Timing of the two operators on either side of the sparse backbone, on the shapes of the reference's own tests
 and of the bench workload's tail:
 
-    python3 deploy3d_amd/opbench.py [--calls 200]      (or python3 -m deploy3d_amd.opbench)
+    python3 bench_ops.py [--calls 200]
 
 * SimpleMeanEncoder: 200 000 points, x y ~ N(0, 50), z ~ N(1, 2), grid [2, *, 41, 1536, 1536]
   (tests/voxel_encoder/test_simple_mean.py:8-15)
@@ -18,7 +18,7 @@ import sys
 
 import torch
 
-sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from deploy3d_amd.bev_densify import bev_densify  # noqa: E402
 from deploy3d_amd.simple_mean import simple_mean_encoder  # noqa: E402
 
@@ -84,7 +84,7 @@ def main():
     ap.add_argument("--calls", type=int, default=200)
     args = ap.parse_args()
     if not torch.cuda.is_available():
-        raise SystemExit("opbench needs a GPU")
+        raise SystemExit("bench_ops.py needs a GPU")
     print(json.dumps(voxelize_case(args.calls)), flush=True)
     for rows, cap, shape, dtype in ((10000, 10000, (2, 2, 128, 128), torch.float32),
                                     (10000, 10000, (2, 2, 128, 128), torch.float16),

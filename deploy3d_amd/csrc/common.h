@@ -95,7 +95,18 @@ struct RbSide {
   bool incrementalFill = false;         // the index tensor still holds the previous pass that used this fillState:
                                         // only the slots that pass used and this one does not are set to -1
   bool masksWritten = false;            // out: this build wrote `masks` (SubM rulebooks with a mirrored table)
+  // One block map per stage: a strided build whose caller passes mapRecords (blockMapBytes() of them) keeps its
+  // finished map of the OUTPUT grid there instead of in the workspace; a SubM build on those outputs (same grid,
+  // rows in rank order, which is how a strided build numbers them) that gets the map back with useSharedMap
+  // skips clearing, marking and scanning a map of its own, and the rank -> row permutation.
+  void* mapRecords = nullptr;
+  uint32_t* mapChunkBase = nullptr;
+  bool useSharedMap = false;
+  bool mapWritten = false;              // out: a strided build left its finished map in mapRecords / mapChunkBase
 };
+
+// Bytes of the block map of g's output grid (records, chunk bases); 0 when the grid takes the hash instead.
+void blockMapBytes(const RbGeom& g, int64_t cap, size_t* records, size_t* chunkBase);
 
 // Builds one rulebook on `stream`.  coors [cap, nd+1]; numActIn device int32.
 // index [3, rowLen] with rowLen = kVol * (cap + 128).  outCoors / numActOut are

@@ -169,6 +169,15 @@ struct RulebookLink {
   // incremental fill: index tensor that holds a complete earlier pass of this operator
   const void* primedIndex = nullptr;
   int64_t primedRowLen = 0;
+  // block map of the output grid, kept for the SubM operators that run on this (strided) operator's outputs
+  bool shareMap = false;          // some SubM operator is linked to these coordinates
+  DeviceBuffer mapRecords, mapChunkBase;
+  bool mapValid = false;
+  const void* mapCoors = nullptr;     // outCoors / numActOut the map belongs to
+  const void* mapNumAct = nullptr;
+  int32_t mapGrid[kMaxSpatial + 1] = {0, 0, 0, 0, 0};
+  int mapNd = 0;
+  int64_t mapRows = 0;
 };
 
 size_t maskEntries(int64_t outRows) { return static_cast<size_t>((outRows + 63) / 64 + 8); }
@@ -232,6 +241,7 @@ struct IdxPlugin final : d3d_plugin {
   bool subM = false, transpose = false;
   bool persistentIndex = false;                  // D3D_OPT_PERSISTENT_INDEX
   std::shared_ptr<RulebookLink> link = std::make_shared<RulebookLink>();  // by-products for linked convolutions
+  std::shared_ptr<RulebookLink> coordSource;     // SubM: record of the strided operator that writes inCoors
 
   int kVol() const {
     int v = 1;
@@ -276,6 +286,7 @@ struct IdxPlugin final : d3d_plugin {
   d3d_plugin* clone() const override {
     auto* c = new IdxPlugin(*this);
     c->link = std::make_shared<RulebookLink>();  // a clone is another node: its own by-products, no links yet
+    c->coordSource.reset();
     c->persistentIndex = false;
     return c;
   }
@@ -447,6 +458,30 @@ struct IdxPlugin final : d3d_plugin {
       side.fillState = static_cast<uint32_t*>(link->fillState.ptr);
       side.incrementalFill = link->primedIndex == outputs[0] && link->primedRowLen == rowLen;
     }
+    // one block map per stage (d3d_link_coords): a strided operator keeps its map for the SubM operators on its
+    // outputs, a SubM operator takes the map of the operator that wrote the coordinates it is handed
+    std::shared_ptr<RulebookLink> source = subM ? coordSource : nullptr;
+    std::unique_lock<std::mutex> sourceLock;
+    if (!subM && link->shareMap && !g_noAlloc) {
+      size_t recBytes = 0, chunkBytes = 0;
+      blockMapBytes(g, cap, &recBytes, &chunkBytes);
+      if (recBytes && link->mapRecords.reserve(recBytes) == D3D_OK && link->mapChunkBase.reserve(chunkBytes) == D3D_OK) {
+        side.mapRecords = link->mapRecords.ptr;
+        side.mapChunkBase = static_cast<uint32_t*>(link->mapChunkBase.ptr);
+      }
+    }
+    link->mapValid = false;
+    if (source && source != link) {
+      sourceLock = std::unique_lock<std::mutex>(source->mutex);
+      bool same = source->mapValid && source->mapCoors == inputs[0] && source->mapNumAct == inputs[1] &&
+                  source->mapNd == nd && source->mapRows == cap;
+      for (int i = 0; same && i <= nd; ++i) same = source->mapGrid[i] == grid[i];
+      if (same) {
+        side.mapRecords = source->mapRecords.ptr;
+        side.mapChunkBase = static_cast<uint32_t*>(source->mapChunkBase.ptr);
+        side.useSharedMap = true;
+      }
+    }
     link->tableValid = link->masksValid = false;
     link->primedIndex = nullptr;
     int32_t rc = launchRulebook(g, subM, static_cast<const int32_t*>(inputs[0]),
@@ -466,6 +501,14 @@ struct IdxPlugin final : d3d_plugin {
       if (side.fillState) {
         link->primedIndex = outputs[0];
         link->primedRowLen = rowLen;
+      }
+      if (side.mapWritten) {
+        link->mapValid = true;
+        link->mapCoors = outputs[2];
+        link->mapNumAct = outputs[3];
+        link->mapNd = nd;
+        link->mapRows = maxNumActOut;
+        for (int i = 0; i <= nd; ++i) link->mapGrid[i] = grid[i];
       }
     }
     return rc;
@@ -1249,6 +1292,31 @@ int32_t d3d_link_rulebook(d3d_plugin* mm, d3d_plugin* idx) {
   int32_t rc = r->wantByProducts(m->cin > 16);
   if (rc != D3D_OK) return rc;
   m->linked = r->link;
+  return D3D_OK;
+  D3D_GUARD_END(D3D_ERR_BAD_ARG)
+}
+
+int32_t d3d_link_coords(d3d_plugin* subm, d3d_plugin* producer) {
+  D3D_GUARD_BEGIN
+  auto* s = dynamic_cast<IdxPlugin*>(subm);
+  if (!s || !s->subM) {
+    setError("d3d_link_coords: the first handle must be a submanifold SPConvIdx{N}d");
+    return D3D_ERR_BAD_ARG;
+  }
+  if (!producer) {
+    s->coordSource.reset();
+    return D3D_OK;
+  }
+  auto* r = dynamic_cast<IdxPlugin*>(producer);
+  if (!r || r->subM || r->nd != s->nd) {
+    setError("d3d_link_coords: the second handle must be a strided or transposed SPConvIdx%dd", s->nd);
+    return D3D_ERR_BAD_ARG;
+  }
+  {
+    std::lock_guard<std::mutex> lock(r->link->mutex);
+    r->link->shareMap = true;
+  }
+  s->coordSource = r->link;
   return D3D_OK;
   D3D_GUARD_END(D3D_ERR_BAD_ARG)
 }

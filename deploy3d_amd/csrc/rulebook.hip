@@ -941,11 +941,8 @@ bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* 
           const BmRecord r = records[rec];
           if ((r.bits >> bit) & 1ull) {
             const uint32_t rank = bmRank(r, bit, chunkBase, rec);
-            if (SUBM) {
-              row[j] = rank;  // the compaction turns ranks into rows through perm[] when rows are shuffled
-            } else if (rank < static_cast<uint32_t>(maxNumActOut)) {
-              row[j] = rank;
-            }
+            if (SUBM ? rank < static_cast<uint32_t>(n) : rank < static_cast<uint32_t>(maxNumActOut))
+              row[j] = rank;  // SubM: the compaction turns ranks into rows through perm[] when rows are shuffled
           }
         }
       }
@@ -1217,11 +1214,8 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
       const unsigned long long bits = (static_cast<unsigned long long>(v.y) << 32) | v.x;
       if ((bits >> bit) & 1ull) {
         const uint32_t rank = v.z + static_cast<uint32_t>(__popcll(bits & ((1ull << bit) - 1ull)));
-        if (SUBM) {
-          row = rank;  // the compaction turns ranks into rows through perm[] when rows are shuffled
-        } else if (rank < static_cast<uint32_t>(maxNumActOut)) {
-          row = rank;
-        }
+        if (SUBM ? rank < static_cast<uint32_t>(n) : rank < static_cast<uint32_t>(maxNumActOut))
+          row = rank;  // SubM: the compaction turns ranks into rows through perm[] when rows are shuffled
       }
     }
     if (inRange) staging[static_cast<int64_t>(tap) * pitch + i] = row;
@@ -1352,7 +1346,8 @@ bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
         const uint32_t bit = (((part1 << m.shift[2]) | part2[q2]) << m.shift[3]) | part3[q3];
         if ((bits >> bit) & 1ull) {
           const uint32_t rank = v.z + static_cast<uint32_t>(__popcll(bits & ((1ull << bit) - 1ull)));
-          if (SUBM || rank < static_cast<uint32_t>(maxNumActOut)) row = rank;
+          // SubM: a rank past the live rows is a cell of a shared map whose row a truncated strided build dropped
+          if (SUBM ? rank < static_cast<uint32_t>(n) : rank < static_cast<uint32_t>(maxNumActOut)) row = rank;
         }
       }
       const int tap = (i1 * K2 + q2) * K3 + q3;
@@ -1518,6 +1513,14 @@ bool blockMapFits(const RbGeom& g) {
 
 }  // namespace
 
+void blockMapBytes(const RbGeom& g, int64_t cap, size_t* records, size_t* chunkBase) {
+  *records = *chunkBase = 0;
+  const RbWorkspace w = planRulebookWorkspace(g, cap, false, ~static_cast<size_t>(0));
+  if (!w.blockMap) return;
+  *records = static_cast<size_t>(w.nRecords) * sizeof(BmRecord);
+  *chunkBase = static_cast<size_t>(w.nChunks > 0 ? w.nChunks : 1) * 4;
+}
+
 size_t rulebookWorkspaceBytes(const RbGeom& g, int64_t cap, bool subM, bool gridKnown) {
   // enough for either structure, so the choice at enqueue time is free
   size_t need = planWith(g, cap, subM, false).total;
@@ -1528,11 +1531,19 @@ size_t rulebookWorkspaceBytes(const RbGeom& g, int64_t cap, bool subM, bool grid
   return need;
 }
 
+// The block map pays for every record of the grid (cleared and scanned on each pass) whatever the number of
+// voxels; with more than kMaxRecordsPerRow records per row of capacity that costs more than the hash saves
+// (measured: 20 000 voxels uniform in a [41,1600,1408] grid, 1.44 M records: 50 us against 36 us on the hash).
+constexpr uint64_t kMaxRecordsPerRow = 32;
+
 RbWorkspace planRulebookWorkspace(const RbGeom& g, int64_t cap, bool subM, size_t workspaceBytes) {
   const int pin = structureOverride();
   if (pin != 1 && blockMapFits(g)) {
+    uint64_t records;
+    makeBlockMap(g, &records);
     const RbWorkspace w = planWith(g, cap, subM, true);
-    if (w.total <= workspaceBytes || pin == 2) return w;
+    if (pin == 2 || (w.total <= workspaceBytes && records <= kMaxRecordsPerRow * static_cast<uint64_t>(cap < 1 ? 1 : cap)))
+      return w;
   }
   return planWith(g, cap, subM, false);
 }
@@ -1628,25 +1639,33 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   if (w.blockMap) {
     uint64_t nRecords64;
     const BlockMap m = makeBlockMap(g, &nRecords64);
-    auto* records = reinterpret_cast<BmRecord*>(ws + w.table);
+    // the map lives in the workspace, or in the caller's buffers that carry it from a strided build to the SubM
+    // builds on its outputs
+    const bool mapOutside = side.mapRecords && side.mapChunkBase && (!subM || side.useSharedMap);
+    const bool sharedMap = subM && mapOutside;
+    auto* records = mapOutside ? static_cast<BmRecord*>(side.mapRecords) : reinterpret_cast<BmRecord*>(ws + w.table);
     auto* perm = reinterpret_cast<uint32_t*>(ws + w.ids);
-    auto* chunkBase = reinterpret_cast<uint32_t*>(ws + w.ownCnt);
+    auto* chunkBase = mapOutside ? side.mapChunkBase : reinterpret_cast<uint32_t*>(ws + w.ownCnt);
+    side.mapWritten = !subM && mapOutside;
     uint32_t* scanTicket = ownTotals + g.kVol + 1;
     const dim3 perChunk(w.nChunks > 0 ? w.nChunks : 1);
     uint32_t* permShuffled = ownTotals + g.kVol;
-    if (subM) {
+    if (subM && !sharedMap) {
       compactPerm = perm;
       compactPermFlag = permShuffled;
     }
     const bool near = nearEligible(g, m);
     const int ksel = near ? fixedKernelShape(g) : 0;
     const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
-    hipLaunchKernelGGL(bmReset, fillGrid(static_cast<int64_t>(w.nRecords) + ((near || incremental) ? 0 : nIndex / 4) + 1), block, 0,
-                       stream, reinterpret_cast<uint4*>(records), static_cast<int64_t>(w.nRecords),
+    const int64_t clearRecords = sharedMap ? 0 : static_cast<int64_t>(w.nRecords);
+    hipLaunchKernelGGL(bmReset, fillGrid(clearRecords + ((near || incremental) ? 0 : nIndex / 4) + 1), block, 0,
+                       stream, reinterpret_cast<uint4*>(records), clearRecords,
                        near ? nullptr : fillIndex, nIndex, cnt,
                        static_cast<int64_t>((w.totals - w.cnt) / 4 + totalsWords(g.kVol, w.nChunks)),
                        numIndex, masks, nMasks, fillState);
-    if (subM) {
+    if (sharedMap) {
+      // the strided build that wrote these coordinates marked and scanned this very grid
+    } else if (subM) {
       hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
     } else if (near) {
       switch (ksel) {
@@ -1660,7 +1679,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       hipLaunchKernelGGL(bmMarkCandidates, perTap, block, 0, stream, g, m, coors, numActIn, cap, records);
     }
     // D3D_RULEBOOK_ORDERED_SCAN=1: acquire-release tickets (see bmScan)
-    if (debugEnv("D3D_RULEBOOK_ORDERED_SCAN"))
+    if (sharedMap) {
+    } else if (debugEnv("D3D_RULEBOOK_ORDERED_SCAN"))
       hipLaunchKernelGGL(bmScan<true>, perChunk, block, 0, stream, records, w.nRecords, chunkBase, w.nChunks, scanTicket,
                          scanTicket + 1, subM ? nullptr : numActOut, maxNumActOut);
     else
@@ -1670,14 +1690,14 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       if (!subM)
         hipLaunchKernelGGL(bmEmitCoords, dim3((w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64)), block, 0, stream,
                            g, m, records, chunkBase, w.nRecords, outCoors, maxNumActOut);
-      if (subM)
+      if (subM && !sharedMap)
         hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, chunkBase,
                            perm, permShuffled);
     }
     if (near) {  // probe workgroups interleaved 1:1 with fill workgroups (index tensor, neighbour table)
       const uint32_t probeBlocks = perInput.x;
       const uint32_t quads = probeBlocks;
-      const uint32_t extra = subM ? probeBlocks : (w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64);
+      const uint32_t extra = sharedMap ? 0u : (subM ? probeBlocks : (w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64));
       const dim3 fused(quads * 2 + extra);
       int32_t* fillB = (nbrOut && nbrRows > 0 && !mirror) ? nbrOut : nullptr;
       const int64_t nFillB = fillB ? static_cast<int64_t>(g.kVol) * nbrRows : 0;

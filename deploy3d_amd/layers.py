@@ -21,8 +21,9 @@ def _round_up(v, m):
 class SparseTensor:
     """Features + coordinates + live count + grid, all at static capacity."""
 
-    def __init__(self, feats, coors, num_act, grid, batch=1):
+    def __init__(self, feats, coors, num_act, grid, batch=1, producer=None):
         self.feats, self.coors, self.num_act, self.grid, self.batch = feats, coors, num_act, list(grid), batch
+        self.producer = producer  # the strided SPConvIdx operator that wrote coors / num_act, if one did
 
     @property
     def capacity(self):
@@ -46,6 +47,7 @@ class Rulebook:
         self.plugin = plugin  # the SPConvIdx operator that wrote it: convolutions of the key link to it
         self.out_coors, self.num_act_out, self.out_grid = out_coors, num_act_out, out_grid
         self.in_coors, self.num_act_in, self.in_grid = in_tensor.coors, in_tensor.num_act, in_tensor.grid
+        self.in_producer = in_tensor.producer
 
 
 class SparseConvLayer:
@@ -81,6 +83,9 @@ class SparseConvLayer:
             ws = torch.empty(max(1, self.idx_plugin.workspace_size(in_descs, out_descs)), dtype=torch.uint8,
                              device=self.device)
             self._idx_state = dict(cap=x.capacity, in_descs=in_descs, out_descs=out_descs, outs=outs, ws=ws)
+            # a SubM rulebook on the outputs of a strided one reuses that operator's occupancy map
+            if self.spec["subm"]:
+                self.idx_plugin.link_coords(x.producer)
         st = self._idx_state
         self.idx_plugin.enqueue(st["in_descs"], st["out_descs"], [x.coors, x.num_act, None], st["outs"], st["ws"])
         outs = st["outs"]
@@ -111,8 +116,9 @@ class SparseConvLayer:
         self.mm_plugin.enqueue(st["in_descs"], st["out_descs"], [feats, num_in, num_out, rb.index, rb.num_index],
                                [st["out"]])
         if inverse:
-            return SparseTensor(st["out"], rb.in_coors, rb.num_act_in, rb.in_grid, x.batch)
-        return SparseTensor(st["out"], rb.out_coors, rb.num_act_out, rb.out_grid, x.batch)
+            return SparseTensor(st["out"], rb.in_coors, rb.num_act_in, rb.in_grid, x.batch, rb.in_producer)
+        return SparseTensor(st["out"], rb.out_coors, rb.num_act_out, rb.out_grid, x.batch,
+                            x.producer if self.spec["subm"] else rb.plugin)
 
 
 class SparseBackbone:
@@ -157,7 +163,7 @@ class SparseBackbone:
                 inp = cur
             elif "+" in src:
                 a, b = (outs[s] for s in src.split("+"))
-                inp = SparseTensor(a.feats + b.feats, a.coors, a.num_act, a.grid, a.batch)
+                inp = SparseTensor(a.feats + b.feats, a.coors, a.num_act, a.grid, a.batch, a.producer)
             else:
                 inp = outs[src]
             inputs[spec["name"]] = inp

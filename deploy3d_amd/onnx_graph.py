@@ -20,7 +20,7 @@ import struct
 
 import torch
 
-from .plugin import OPT_PERSISTENT_INDEX, Plugin, TensorDesc
+from .plugin import OPT_PERSISTENT_INDEX, EngineError, Plugin, TensorDesc
 
 # onnx.TensorProto.DataType
 FLOAT, INT8, INT32, FLOAT16, BFLOAT16 = 1, 3, 6, 10, 16
@@ -345,6 +345,14 @@ class GraphExecutor:
                 continue
             if p.name.startswith("SPConvIdx"):
                 p.set_option(OPT_PERSISTENT_INDEX, 1)  # the executor owns the index tensor and nobody else writes it
+                # a SubM node on the coordinates a strided node wrote reuses that node's occupancy map
+                src = producer.get(n.inputs[0])
+                if src is not None and src[1] == 2 and producer.get(n.inputs[1]) == (src[0], 3) and \
+                        src[0] in self.plugins and self.plugins[src[0]].name == p.name:
+                    try:
+                        p.link_coords(self.plugins[src[0]])
+                    except EngineError:
+                        pass  # this node is not submanifold
             if p.name == "SPConvMM" and len(n.inputs) >= 5:
                 src = producer.get(n.inputs[3])
                 if src is not None and src[1] == 0 and src[0] in self.plugins and \

@@ -27,7 +27,7 @@ EXPORTS = [
     "d3d_create", "d3d_clone", "d3d_destroy", "d3d_plugin_type", "d3d_plugin_version", "d3d_serialize_size",
     "d3d_serialize", "d3d_num_outputs", "d3d_output_dims", "d3d_output_dtype", "d3d_supports_format",
     "d3d_configure", "d3d_workspace_size", "d3d_enqueue", "d3d_last_error", "d3d_num_ops", "d3d_op_name",
-    "d3d_enqueue_static", "d3d_link_rulebook", "d3d_set_option",
+    "d3d_enqueue_static", "d3d_link_rulebook", "d3d_link_coords", "d3d_set_option",
 ]
 OPT_PERSISTENT_INDEX = 1
 
@@ -111,6 +111,8 @@ def load_library(path=None):
     lib.d3d_op_name.argtypes = [i32]
     lib.d3d_link_rulebook.restype = i32
     lib.d3d_link_rulebook.argtypes = [vp, vp]
+    lib.d3d_link_coords.restype = i32
+    lib.d3d_link_coords.argtypes = [vp, vp]
     lib.d3d_set_option.restype = i32
     lib.d3d_set_option.argtypes = [vp, i32, ctypes.c_int64]
     _lib = lib
@@ -204,6 +206,11 @@ class Plugin:
         """SPConvMM only: this node's index tensor is the output of ``idx_plugin`` (None removes the link), so the
         rulebook operator writes the neighbour table and tile masks itself and this node uses them."""
         _check(self._lib.d3d_link_rulebook(self._h, None if idx_plugin is None else idx_plugin._h))
+
+    def link_coords(self, producer):
+        """Submanifold SPConvIdx only: the coordinates it is handed are the output of the strided SPConvIdx
+        ``producer`` (None removes the link), whose occupancy map it then reuses instead of building its own."""
+        _check(self._lib.d3d_link_coords(self._h, None if producer is None else producer._h))
 
     def set_option(self, option, value):
         _check(self._lib.d3d_set_option(self._h, int(option), int(value)))

@@ -172,6 +172,51 @@ def test_single_voxel_and_full_block(engine):
     assert live.sum() == expected
 
 
+def test_submanifold_on_a_strided_operators_map(engine):
+    """d3d_link_coords: a SubM operator on the outputs of a strided operator takes over that operator's occupancy map
+    (no clearing, marking, scanning, no permutation).  Its index tensor must equal, bit for bit, the oracle's for
+    those coordinates and what the same operator builds on its own - also when the strided operator truncated its
+    outputs (the map then holds cells whose rows were dropped) and when the tensors handed over are not the ones
+    the strided operator wrote (the link must not be used)."""
+    import torch
+    from deploy3d_amd import spconv_index_nd
+    from deploy3d_amd.spconv_index import index_plugin
+    grid, n = (12, 40, 33), 3000
+    rng = np.random.default_rng(99)
+    coords = random_cloud(rng, n, grid, 1)
+    c = torch.from_numpy(coords).cuda()
+    num = torch.tensor([n], dtype=torch.int32, device="cuda")
+    shape = torch.empty((1, 0) + grid, dtype=torch.int32, device="cuda")
+    down = ((3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1), (0, 0, 0))
+    same = ((3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), (0, 0, 0))
+    for max_out in (8 * n, 700):
+        producer = index_plugin(*down, max_out, False, False)
+        subm = index_plugin(*same, max_out, True, False)
+        results = []
+        for linked in (True, False, True):
+            subm.link_coords(producer if linked else None)
+            _, _, out_coors, num_out, out_shape = spconv_index_nd(c, num, shape, *down, max_out, False, False)
+            index, num_index = spconv_index_nd(out_coors, num_out, out_shape, *same, max_out, True, False)
+            torch.cuda.synchronize()
+            results.append(index.cpu().numpy())
+            m = int(num_out.item())
+            ref = oracle.rulebook(out_coors.cpu().numpy(), m, (1,) + tuple(out_shape.shape[2:]), *same[:4], max_out, True)
+            assert int(num_index.item()) == ref["num_index"]
+            np.testing.assert_array_equal(results[-1], ref["index"])
+        np.testing.assert_array_equal(results[0], results[1])
+        # other coordinates in a tensor the producer did not write: the link is there, the map must not be used
+        subm.link_coords(producer)
+        other = torch.zeros_like(out_coors)
+        m2 = min(500, max_out)
+        other[:m2] = torch.from_numpy(random_cloud(rng, m2, tuple(out_shape.shape[2:]), 1)).cuda()
+        num2 = torch.tensor([m2], dtype=torch.int32, device="cuda")
+        index, num_index = spconv_index_nd(other, num2, out_shape, *same, max_out, True, False)
+        torch.cuda.synchronize()
+        ref = oracle.rulebook(other.cpu().numpy(), m2, (1,) + tuple(out_shape.shape[2:]), *same[:4], max_out, True)
+        np.testing.assert_array_equal(index.cpu().numpy(), ref["index"])
+        subm.link_coords(None)
+
+
 def test_ordered_scan_variant(engine, monkeypatch):
     """D3D_RULEBOOK_ORDERED_SCAN=1 selects acquire-release tickets in the scan pass of the block map: same results."""
     monkeypatch.setenv("D3D_RULEBOOK_ORDERED_SCAN", "1")
