@@ -12,6 +12,8 @@
 // atomics, and a bit-reproducible result.
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace d3d {
@@ -175,6 +177,96 @@ int32_t launchNarrow(const ConvArgs& a, hipStream_t stream) {
   return D3D_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Narrow layers proper (at most 32 input and 32 output channels, any storage type; fp32 math): lanes across the
+// output channels, several rows per wavefront.  A wavefront holds 64 / CP rows at a time (CP = 16 or 32 lanes per
+// row); lane (r, co) accumulates channel co of row r over all taps and input channels.  The 16 or 32 lanes of a
+// row read the same input values - one address per row, served as a broadcast, 128 bits at a time when the rows
+// allow it - and consecutive LDS words of the weight slice W[tap][ci][:], which every row shares; a tap that none
+// of the wavefront's rows has is skipped after one ballot, and the table entries of 27 taps are requested
+// together so that their latencies overlap.  Nothing is staged per tap and there is no barrier after the weights
+// have landed: such a layer moves a few megabytes, and what it costs is the chain of dependent loads.
+// ---------------------------------------------------------------------------
+template <class T, int CP>
+__global__ void __launch_bounds__(kConvThreads)
+convNarrowRows(const T* __restrict__ in, T* __restrict__ out, const float* __restrict__ w, const float* __restrict__ bias,
+               const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror, int kVol, int cin, int cout,
+               int64_t inRows, int64_t outRows, int relu, int rowsPerWave) {
+  extern __shared__ __attribute__((aligned(16))) float wl[];  // [kVol][cin][CP], channels past cout zero
+  const int total = kVol * cin * CP;
+  for (int e = threadIdx.x; e < total; e += kConvThreads) {
+    const int co = e % CP, tc = e / CP;
+    wl[e] = co < cout ? w[static_cast<size_t>(tc) * cout + co] : 0.f;
+  }
+  __syncthreads();
+  constexpr int RP = 64 / CP;
+  constexpr int kBatch = 27;  // table entries requested together: a whole 3x3x3 kernel
+  const int lane = threadIdx.x & 63, r = lane / CP, co = lane % CP;
+  const int64_t first = (static_cast<int64_t>(blockIdx.x) * (kConvThreads / 64) + (threadIdx.x >> 6)) * rowsPerWave;
+  const float b = (bias && co < cout) ? bias[co] : 0.f;
+  const bool wide = std::is_same<T, float>::value && (cin & 3) == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
+  for (int64_t row0 = first; row0 < first + rowsPerWave && row0 < outRows; row0 += RP) {
+    const int64_t row = row0 + r;
+    const bool valid = row < outRows;
+    float acc = b;
+    for (int tap0 = 0; tap0 < kVol; tap0 += kBatch) {
+      int32_t ids[kBatch];
+#pragma unroll
+      for (int q = 0; q < kBatch; ++q) {
+        const int tap = tap0 + q;
+        ids[q] = (valid && tap < kVol) ? nbr[static_cast<int64_t>(tapMirror ? kVol - 1 - tap : tap) * nbrPitch + row] : -1;
+      }
+#pragma unroll
+      for (int q = 0; q < kBatch; ++q) {
+        const int32_t idx = ids[q];
+        const bool has = idx >= 0 && idx < inRows;
+        if (__ballot(has) == 0ull) continue;  // wavefront-uniform
+        if (has) {
+          const float* wt = wl + static_cast<size_t>(tap0 + q) * cin * CP + co;
+          const T* x = in + static_cast<size_t>(idx) * cin;
+          if (wide) {
+            for (int ci = 0; ci < cin; ci += 4) {
+              const float4v v = *reinterpret_cast<const float4v*>(reinterpret_cast<const float*>(x) + ci);
+              acc = __builtin_fmaf(v[0], wt[(ci + 0) * CP], acc);
+              acc = __builtin_fmaf(v[1], wt[(ci + 1) * CP], acc);
+              acc = __builtin_fmaf(v[2], wt[(ci + 2) * CP], acc);
+              acc = __builtin_fmaf(v[3], wt[(ci + 3) * CP], acc);
+            }
+          } else {
+            for (int ci = 0; ci < cin; ++ci) acc = __builtin_fmaf(Elem<T>::load(x + ci), wt[ci * CP], acc);
+          }
+        }
+      }
+    }
+    if (relu) acc = acc > 0.f ? acc : 0.f;
+    if (valid && co < cout) Elem<T>::store(out + static_cast<size_t>(row) * cout + co, acc);
+  }
+}
+
+template <class T>
+int32_t launchNarrowRows(const ConvArgs& a, hipStream_t stream) {
+  const int cp = a.cout <= 16 ? 16 : 32;
+  const size_t lds = static_cast<size_t>(a.kVol) * a.cin * cp * sizeof(float);
+  if (a.cin > 32 || a.cout > 32 || lds > 64 * 1024) return D3D_ERR_UNSUPPORTED;
+  // Small layers: one group of rows per wavefront - the layer is a chain of dependent loads per row, and only many
+  // wavefronts hide it (20 000 rows: 22 us at 16 rows per wavefront, 14 us at 4).  Large ones: 16 rows per
+  // wavefront, so that the copy of the weights into LDS is shared by more rows.
+  const bool large = a.outRows > (1 << 16);
+  const int rowsPerWave = large ? 16 : 64 / cp;
+  const int64_t rowsPerBlock = static_cast<int64_t>(rowsPerWave) * (kConvThreads / 64);
+  const dim3 grid(static_cast<unsigned>((a.outRows + rowsPerBlock - 1) / rowsPerBlock));
+  const int64_t pitch = a.nbrPitch > 0 ? a.nbrPitch : a.outRows;
+  if (cp == 16)
+    hipLaunchKernelGGL((convNarrowRows<T, 16>), grid, dim3(kConvThreads), lds, stream,
+                       static_cast<const T*>(a.in), static_cast<T*>(a.out), a.weightsF32, a.bias, a.nbr, pitch,
+                       a.tapMirror, a.kVol, a.cin, a.cout, a.inRows, a.outRows, a.relu, rowsPerWave);
+  else
+    hipLaunchKernelGGL((convNarrowRows<T, 32>), grid, dim3(kConvThreads), lds, stream,
+                       static_cast<const T*>(a.in), static_cast<T*>(a.out), a.weightsF32, a.bias, a.nbr, pitch,
+                       a.tapMirror, a.kVol, a.cin, a.cout, a.inRows, a.outRows, a.relu, rowsPerWave);
+  return D3D_OK;
+}
+
 bool isMfmaChannels(int c) { return c == 16 || c == 32 || c == 64 || c == 128; }
 
 // rows of `inBytes` bytes widened to `outBytes` (a multiple of 16) with zeros, so that a narrow first layer
@@ -269,10 +361,21 @@ int32_t launchConv(const ConvArgs& a, hipStream_t stream) {
       rc = a.dtype == D3D_HALF ? launchNarrow<_Float16>(b, stream) : launchNarrow<__bf16>(b, stream);
     }
   } else {
+    const char* rowsEnv = debugEnv("D3D_CONV_NARROW_ROWS");  // =0: keep the tile kernel (tests)
+    const bool rows = !(rowsEnv && rowsEnv[0] == '0');
     switch (a.dtype) {
-      case D3D_FLOAT: rc = launchNarrow<float>(a, stream); break;
-      case D3D_HALF: rc = launchNarrow<_Float16>(a, stream); break;
-      case D3D_BF16: rc = launchNarrow<__bf16>(a, stream); break;
+      case D3D_FLOAT:
+        rc = rows ? launchNarrowRows<float>(a, stream) : D3D_ERR_UNSUPPORTED;
+        if (rc == D3D_ERR_UNSUPPORTED) rc = launchNarrow<float>(a, stream);
+        break;
+      case D3D_HALF:
+        rc = rows ? launchNarrowRows<_Float16>(a, stream) : D3D_ERR_UNSUPPORTED;
+        if (rc == D3D_ERR_UNSUPPORTED) rc = launchNarrow<_Float16>(a, stream);
+        break;
+      case D3D_BF16:
+        rc = rows ? launchNarrowRows<__bf16>(a, stream) : D3D_ERR_UNSUPPORTED;
+        if (rc == D3D_ERR_UNSUPPORTED) rc = launchNarrow<__bf16>(a, stream);
+        break;
       default: setError("conv: dtype %d not implemented", a.dtype); return D3D_ERR_UNSUPPORTED;
     }
   }

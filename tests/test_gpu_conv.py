@@ -94,6 +94,18 @@ def test_narrow_subm(engine, cin, cout, dtype):
     run_case(2500, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, dtype, True, relu=(cout == 16))
 
 
+@pytest.mark.parametrize("cin,cout,dtype", [(5, 16, "float16"), (16, 16, "float32"), (3, 7, "float32"), (24, 32, "float32"),
+                                            (32, 20, "bfloat16")])
+def test_narrow_tile_kernel_still_matches(engine, monkeypatch, cin, cout, dtype):
+    """Layers of at most 32 x 32 channels take the rows-per-wavefront kernel; D3D_CONV_NARROW_ROWS=0 keeps them on the
+    tile kernel that serves every other shape.  Both against the oracle."""
+    monkeypatch.setenv("D3D_CONV_NO_PAD", "1")  # keep 2-byte layers off the MFMA path
+    run_case(2500, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, dtype, True, seed=41)
+    run_case(2500, (10, 36, 30), (3, 3, 3), (2, 2, 2), (1, 1, 1), cin, cout, dtype, False, seed=42, relu=True)
+    monkeypatch.setenv("D3D_CONV_NARROW_ROWS", "0")
+    run_case(2500, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, dtype, True, seed=41)
+
+
 def test_narrow_strided_fp32(engine):
     run_case(2500, (10, 36, 30), (3, 3, 3), (2, 2, 2), (1, 1, 1), 16, 16, "float32", False)
 
