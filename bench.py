@@ -29,7 +29,9 @@ ELEM = {"float16": 2, "bfloat16": 2, "int8": 1, "float32": 4}
 # 256 MiB copy of --pmc-copy-mib (FETCH_SIZE reads half the copied KiB: factor 2.0; WRITE_SIZE factor 1.0).
 # A cached reading: it belongs to the kernel and workload named here and is null for any other.
 TRAFFIC_SOURCE = "profiles/config3_backbone_hbm_traffic_pmc.txt"
-MEASURED_TRAFFIC = {(3, 120000, "conv3_1"): None}
+# conv3_0 / conv3_1 run the same kernel on the same rulebook: FETCH_SIZE 46159 and WRITE_SIZE 34464 per dispatch.
+MEASURED_TRAFFIC = {(3, 120000, "conv3_0"): int((46159 * 2.0 + 34464 * 1.0) * 1024),
+                    (3, 120000, "conv3_1"): int((46159 * 2.0 + 34464 * 1.0) * 1024)}
 DEFAULT_VOXELS = {1: 20000, 2: 60000, 3: 120000, 4: 120000, 5: 250000}
 WORKLOAD = {
     1: "config 1: one SubM 3x3x3 16->16, fp32, %d voxels uniform in grid [41,1600,1408]",
@@ -205,6 +207,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="time eager enqueues instead of HIP-graph replays")
     ap.add_argument("--no-overlap", action="store_true",
                     help="enqueue rulebooks and convolutions on one stream instead of three")
+    ap.add_argument("--no-op-timing", action="store_true",
+                    help="skip the per-operator graphs and the rooflines built on them (counter runs, where every "
+                         "extra dispatch is profiled)")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="end with ONE device-to-device copy of this many MiB: the dispatch of known size that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this script")
@@ -273,6 +278,8 @@ def main():
         layer_ms, rulebook_ms = [], {}
         first_of_key = {}
         for li, (spec, lyr) in enumerate(zip(specs, net.layers)):
+            if args.no_op_timing:
+                break
             inp = net.inputs[spec["name"]]
             if spec["key"] not in first_of_key:
                 first_of_key[spec["key"]] = li
@@ -327,7 +334,7 @@ def main():
                      "int8": peaks.get("mfma_i8_tops")}.get(cfg["dtype"])
         meas_hbm = peaks.get("hbm_copy_gbs")
     rooflines = []
-    for li, spec in enumerate(specs):
+    for li, spec in enumerate(specs[:len(layer_ms)]):
         key = spec["key"]
         kvol = int(np.prod(spec["ksize"]))
         secs = layer_ms[li] * 1e-3
@@ -369,11 +376,13 @@ def main():
         rooflines.append(r)
     # dominant kernel: the MFMA convolution with the largest device time; a configuration without one (config 1) is
     # judged on its slowest operator
-    mfma = [r for r in rooflines if r["bound"] == "mfma"]
-    roofline = dict(max(mfma or rooflines, key=lambda r: r["avg_launch_ms"]))
-    roofline["traffic_source"] = TRAFFIC_SOURCE if roofline.get("traffic") else None
-    if meas_mfma and roofline["bound"] == "mfma":
-        roofline["measured_peak"] = meas_mfma
+    roofline = None
+    if rooflines:
+        mfma = [r for r in rooflines if r["bound"] == "mfma"]
+        roofline = dict(max(mfma or rooflines, key=lambda r: r["avg_launch_ms"]))
+        roofline["traffic_source"] = TRAFFIC_SOURCE if roofline.get("traffic") else None
+        if meas_mfma and roofline["bound"] == "mfma":
+            roofline["measured_peak"] = meas_mfma
 
     out = {
         "metric": METRIC, "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,

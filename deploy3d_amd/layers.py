@@ -138,6 +138,11 @@ class SparseBackbone:
         self.specs = layers
         self.layers = [SparseConvLayer(s, w, b, cap, dtype=dtype, device=device)
                        for s, (w, b), cap in zip(layers, weights, capacities)]
+        # every convolution reads the rulebook of the first layer that names its indice key: link them now, so
+        # that already the first pass has the rulebook operators write the tables
+        owner = {}
+        for spec, lyr in zip(layers, self.layers):
+            lyr.mm_plugin.link_rulebook(owner.setdefault(spec["key"], lyr).idx_plugin)
         self.overlap = overlap
         self._side = None
 
