@@ -207,6 +207,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="time eager enqueues instead of HIP-graph replays")
     ap.add_argument("--no-overlap", action="store_true",
                     help="enqueue rulebooks and convolutions on one stream instead of three")
+    ap.add_argument("--no-fused", action="store_true", help="skip the second figure (index tensors unwritten)")
     ap.add_argument("--no-op-timing", action="store_true",
                     help="skip the per-operator graphs and the rooflines built on them (counter runs, where every "
                          "extra dispatch is profiled)")
@@ -314,6 +315,35 @@ def main():
             ms = (time.perf_counter() - t0) * 1e3 / args.steps
             mode = "hip-graph replay" + streams
         same = bool(torch.equal(y.feats, ref_out))
+        # second figure: the same pass by a runner that declares itself the only reader of the index tensors
+        # (D3D_OPT_INDEX_UNUSED): rulebook operators write the tables their linked convolutions read and leave the
+        # reference-format index tensors unwritten.  Not `value`: the operators' documented outputs are incomplete.
+        fused = None
+        if not args.no_graph and not args.no_fused:
+            net2 = layers.SparseBackbone(specs, weights, caps, dtype=dtype, overlap=not args.no_overlap,
+                                         index_tensors=False)
+            for _ in range(2):
+                y2 = net2.forward(x)
+            stream.synchronize()
+            graph2 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph2, stream=stream):
+                y2 = net2.forward(x)
+            for _ in range(2):
+                graph2.replay()
+            stream.synchronize()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                graph2.replay()
+            torch.cuda.synchronize()
+            ms2 = (time.perf_counter() - t0) * 1e3 / args.steps
+            n2 = int(y2.num_act.item())
+            fused = {"ms_per_step": round(ms2, 4), "effective_tflops": round(total_flops / (ms2 * 1e-3) / 1e12, 2),
+                     "what": "same pass with D3D_OPT_INDEX_UNUSED on every rulebook operator: index tensors left "
+                             "unwritten, tables and tile masks written by the probe pass, no compaction",
+                     "outputs_equal_full_pass": bool(n2 == int(y.num_act.item()) and torch.equal(y2.feats, y.feats)
+                                                     and torch.equal(y2.coors[:n2], y.coors[:n2]))}
+            del net2, graph2
         n_final = int(y.num_act.item())
         gpu_coords = y.coors[:n_final].cpu().numpy()
         gpu_feats = y.feats[:n_final].float().cpu().numpy() if dtype != torch.int8 else y.feats[:n_final].cpu().numpy()
@@ -399,6 +429,7 @@ def main():
         "outputs_match_warmup": same,
         "layer_ms": {s["name"]: round(t, 4) for s, t in zip(specs, layer_ms)},
         "rulebook_ms": {k: round(t, 4) for k, t in rulebook_ms.items()},
+        "index_unused": fused,
         "roofline": roofline,
         "rooflines": rooflines,
         "measured_peak": peaks,

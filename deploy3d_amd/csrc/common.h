@@ -95,6 +95,10 @@ struct RbSide {
   bool incrementalFill = false;         // the index tensor still holds the previous pass that used this fillState:
                                         // only the slots that pass used and this one does not are set to -1
   bool masksWritten = false;            // out: this build wrote `masks` (SubM rulebooks with a mirrored table)
+  bool skipIndex = false;               // nothing reads the index tensor but convolutions that read nbr: where the
+                                        // build can write nbr (and masks) without compacting, it leaves the index
+                                        // tensor unwritten (numIndex is still written)
+  bool indexWritten = true;             // out: false when skipIndex was honoured
   // One block map per stage: a strided build whose caller passes mapRecords (blockMapBytes() of them) keeps its
   // finished map of the OUTPUT grid there instead of in the workspace; a SubM build on those outputs (same grid,
   // rows in rank order, which is how a strided build numbers them) that gets the map back with useSharedMap

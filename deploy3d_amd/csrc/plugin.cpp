@@ -240,6 +240,7 @@ struct IdxPlugin final : d3d_plugin {
   int32_t maxNumActOut = 0;
   bool subM = false, transpose = false;
   bool persistentIndex = false;                  // D3D_OPT_PERSISTENT_INDEX
+  bool indexUnused = false;                      // D3D_OPT_INDEX_UNUSED
   std::shared_ptr<RulebookLink> link = std::make_shared<RulebookLink>();  // by-products for linked convolutions
   std::shared_ptr<RulebookLink> coordSource;     // SubM: record of the strided operator that writes inCoors
 
@@ -288,6 +289,7 @@ struct IdxPlugin final : d3d_plugin {
     c->link = std::make_shared<RulebookLink>();  // a clone is another node: its own by-products, no links yet
     c->coordSource.reset();
     c->persistentIndex = false;
+    c->indexUnused = false;
     return c;
   }
   int32_t numOutputs() const override { return subM ? 2 : 5; }  // index_trt.cu:98-101
@@ -307,6 +309,12 @@ struct IdxPlugin final : d3d_plugin {
   }
 
   int32_t setOption(int32_t option, int64_t value) override {
+    if (option == D3D_OPT_INDEX_UNUSED) {
+      std::lock_guard<std::mutex> lock(link->mutex);
+      indexUnused = value != 0;
+      link->primedIndex = nullptr;
+      return D3D_OK;
+    }
     if (option != D3D_OPT_PERSISTENT_INDEX) return d3d_plugin::setOption(option, value);
     std::lock_guard<std::mutex> lock(link->mutex);
     if (value) {
@@ -454,6 +462,7 @@ struct IdxPlugin final : d3d_plugin {
         side.nMasks = static_cast<int64_t>(maskEntries(maxNumActOut));
       }
     }
+    side.skipIndex = indexUnused && withTable;
     if (persistentIndex && link->fillState.ptr) {
       side.fillState = static_cast<uint32_t*>(link->fillState.ptr);
       side.incrementalFill = link->primedIndex == outputs[0] && link->primedRowLen == rowLen;
@@ -498,7 +507,7 @@ struct IdxPlugin final : d3d_plugin {
       link->rowLen = rowLen;
       link->tableValid = withTable;
       link->masksValid = withTable && side.masksWritten;
-      if (side.fillState) {
+      if (side.fillState && side.indexWritten) {
         link->primedIndex = outputs[0];
         link->primedRowLen = rowLen;
       }

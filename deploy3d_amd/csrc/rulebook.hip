@@ -490,7 +490,7 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
           const uint32_t* __restrict__ totals, int32_t* __restrict__ gather, int32_t* __restrict__ scatter,
           int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* nbr, int64_t nbrRows,
           const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int mirror, int inPlace,
-          unsigned long long* __restrict__ masks, uint32_t* fillState, int incrementalFill) {
+          unsigned long long* __restrict__ masks, uint32_t* fillState, int incrementalFill, int skipIndex) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int tap = blockIdx.y;
   const uint32_t b = blockIdx.x;
@@ -499,6 +499,21 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
     for (int t = 0; t < kVol; ++t) end += tapSegment(totals, t);
     *numIndex = static_cast<int32_t>(end);
     if (fillState) fillState[1] = end;  // what this pass uses of the index tensor: the next pass clears from here
+  }
+  if (skipIndex) {
+    // Nobody reads the index tensor and the probe pass has written table and masks: what is left is turning ranks
+    // into rows where the inputs were not in rank order (in place, in the rows of the mirrored table).
+    if (!(mirror && inPlace && perm && *permShuffled)) return;  // grid-uniform
+    const int64_t at = static_cast<int64_t>(b) * kRbChunk + threadIdx.x * kRbItems;
+    if (at >= liveCount(numActIn, cap)) return;
+    uint4* cell = reinterpret_cast<uint4*>(const_cast<uint32_t*>(staging) + static_cast<int64_t>(tap) * pitch + at);
+    uint4 v = *cell;
+    if (v.x != kNone) v.x = perm[v.x];
+    if (v.y != kNone) v.y = perm[v.y];
+    if (v.z != kNone) v.z = perm[v.z];
+    if (v.w != kNone) v.w = perm[v.w];
+    *cell = v;
+    return;
   }
   // The index tensor still holds the previous pass (of this operator, at this address): instead of clearing it at
   // capacity, write -1 where that pass had entries and this one has none - behind the new end up to the old one,
@@ -1253,7 +1268,13 @@ bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
              uint32_t* __restrict__ perm, uint32_t* permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
              uint32_t* cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
              int64_t nFillB, uint32_t fillBlocks, uint32_t probeBlocks, int32_t* __restrict__ outCoors,
-             uint32_t nRecords) {
+             uint32_t nRecords, unsigned long long* __restrict__ maskOut, int fixTail, int32_t* __restrict__ nbrDirect,
+             int64_t nbrRows) {
+  // Besides the staging entries the pass can write what a linked convolution reads, so that a build whose index
+  // tensor nobody reads needs no compaction: maskOut (SubM, staging rows = rows of the mirrored table) takes the
+  // tile masks - a wavefront's 64 inputs are one 64-row tile - and fixTail has the rows between the live count
+  // and the capacity set to -1; nbrDirect (strided) takes the pairs straight into the scattered table
+  // nbrDirect[tap][output row] = input row, filled with -1 by the reset pass, and nothing is staged.
   constexpr int KP = K2 * K3;
   __shared__ uint4 group[4 * kRbThreads];
   __shared__ uint32_t ldsCnt[KP];
@@ -1280,11 +1301,18 @@ bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
   const uint32_t probeBlock = pidx / K1;
   const int n = liveCount(numActIn, cap);
   const int64_t i0 = static_cast<int64_t>(probeBlock) * kRbThreads;
-  if (i0 >= n) return;  // workgroup-uniform
-  if (threadIdx.x < KP) ldsCnt[threadIdx.x] = 0;
   const int64_t i = i0 + threadIdx.x;
-  const bool inRange = i < n;   // rows below the live count get a staging entry, in the grid or not
-  bool live = inRange;
+  if (i0 >= n) {  // workgroup-uniform
+    if (fixTail && i < cap) {
+#pragma unroll
+      for (int q = 0; q < KP; ++q) staging[static_cast<int64_t>(i1 * KP + q) * pitch + i] = kNone;
+    }
+    return;
+  }
+  if (threadIdx.x < KP) ldsCnt[threadIdx.x] = 0;
+  // rows below the live count get a staging entry, in the grid or not (fixTail: every row below the capacity)
+  const bool inRange = i < n || (fixTail && i < cap);
+  bool live = i < n;
   int c[5] = {0, 0, 0, 0, 0};   // (b, z, y, x) in c[0], c[2..4]; c[1] is the degenerate dim
   if (live && !loadInput(g, coors, i, c)) {
     live = false;
@@ -1333,6 +1361,7 @@ bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
   }
   __syncthreads();  // ldsCnt zeroed
   uint32_t mine = 0;  // lane t of a wavefront counts the wavefront's pairs of tap i1 * KP + t
+  unsigned long long tileBits = 0;  // wavefront-uniform: (mirrored) taps that some input of the wavefront has
   const int lane = threadIdx.x & 63;
 #pragma unroll
   for (int q2 = 0; q2 < K2; ++q2)
@@ -1351,10 +1380,17 @@ bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
         }
       }
       const int tap = (i1 * K2 + q2) * K3 + q3;
-      if (inRange) staging[static_cast<int64_t>(tap) * pitch + i] = row;
+      if (nbrDirect) {
+        if (row != kNone && row < static_cast<uint64_t>(nbrRows))
+          nbrDirect[static_cast<int64_t>(tap) * nbrRows + row] = static_cast<int32_t>(i);
+      } else if (inRange) {
+        staging[static_cast<int64_t>(tap) * pitch + i] = row;
+      }
       const uint32_t hits = static_cast<uint32_t>(__popcll(__ballot(row != kNone)));
       if (lane == q2 * K3 + q3) mine += hits;
+      if (hits) tileBits |= 1ull << ((g.kVol - 1 - tap) & 63);
     }
+  if (maskOut && lane == 0 && tileBits) atomicOr(&maskOut[(i0 + (threadIdx.x & ~63)) >> 6], tileBits);
   if (mine) atomicAdd(&ldsCnt[lane], mine);
   __syncthreads();
   const uint32_t chunk = probeBlock / kRbItems;
@@ -1533,7 +1569,8 @@ size_t rulebookWorkspaceBytes(const RbGeom& g, int64_t cap, bool subM, bool grid
 
 // The block map pays for every record of the grid (cleared and scanned on each pass) whatever the number of
 // voxels; with more than kMaxRecordsPerRow records per row of capacity that costs more than the hash saves
-// (measured: 20 000 voxels uniform in a [41,1600,1408] grid, 1.44 M records: 50 us against 36 us on the hash).
+// (measured: 20 000 voxels uniform in a [41,1600,1408] grid, 1.44 M records, 72 per row: 50 us against 36 us on
+// the hash; 120 000 LiDAR voxels in [41,1440,1440], 1.33 M records, 11 per row: 63 us against 93 us).
 constexpr uint64_t kMaxRecordsPerRow = 32;
 
 RbWorkspace planRulebookWorkspace(const RbGeom& g, int64_t cap, bool subM, size_t workspaceBytes) {
@@ -1634,6 +1671,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   const int64_t nMasks = masks ? side.nMasks : 0;
   side.masksWritten = masks != nullptr;
   bool nbrFilled = mirror;
+  bool skipIndex = false;                     // set below when side.skipIndex can be honoured
+  unsigned long long* compactMasks = masks;   // null when the probe pass writes the masks itself
   const uint32_t* compactPerm = nullptr;      // block-map SubM: staging holds ranks, rows = perm[rank] when shuffled
   const uint32_t* compactPermFlag = nullptr;
   if (w.blockMap) {
@@ -1657,10 +1696,21 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     const bool near = nearEligible(g, m);
     const int ksel = near ? fixedKernelShape(g) : 0;
     const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
+    // A build whose index tensor nobody reads (side.skipIndex) writes table and masks in the probe pass and skips
+    // the compaction: for the kernel shapes of the plane probe, a SubM build with the mirrored table staged in
+    // place, or a strided build with a table to scatter into (which the reset pass then fills with -1, since the
+    // probe pass writes entries into it).
+    skipIndex = side.skipIndex && near && ksel != 0 && nbrOut && (subM ? (mirror && inPlace) : true);
+    const bool directScatter = skipIndex && !subM;
+    const bool probeMasks = subM && mirror && masks && near && ksel != 0;
+    if (probeMasks) compactMasks = nullptr;
+    side.indexWritten = !skipIndex;
+    int32_t* const resetFill = directScatter ? nbrOut : ((near || skipIndex) ? nullptr : fillIndex);
+    const int64_t resetFillN = directScatter ? static_cast<int64_t>(g.kVol) * nbrRows : nIndex;
     const int64_t clearRecords = sharedMap ? 0 : static_cast<int64_t>(w.nRecords);
-    hipLaunchKernelGGL(bmReset, fillGrid(clearRecords + ((near || incremental) ? 0 : nIndex / 4) + 1), block, 0,
+    hipLaunchKernelGGL(bmReset, fillGrid(clearRecords + (resetFill ? resetFillN / 4 : 0) + 1), block, 0,
                        stream, reinterpret_cast<uint4*>(records), clearRecords,
-                       near ? nullptr : fillIndex, nIndex, cnt,
+                       resetFill, resetFillN, cnt,
                        static_cast<int64_t>((w.totals - w.cnt) / 4 + totalsWords(g.kVol, w.nChunks)),
                        numIndex, masks, nMasks, fillState);
     if (sharedMap) {
@@ -1699,7 +1749,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       const uint32_t quads = probeBlocks;
       const uint32_t extra = sharedMap ? 0u : (subM ? probeBlocks : (w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64));
       const dim3 fused(quads * 2 + extra);
-      int32_t* fillB = (nbrOut && nbrRows > 0 && !mirror) ? nbrOut : nullptr;
+      int32_t* fillB = (nbrOut && nbrRows > 0 && !mirror && !directScatter) ? nbrOut : nullptr;
+      int32_t* const probeFillIndex = skipIndex ? nullptr : fillIndex;
       const int64_t nFillB = fillB ? static_cast<int64_t>(g.kVol) * nbrRows : 0;
       nbrFilled = true;
 #define D3D_LAUNCH_PROBE_NEAR(SUBM, KSEL)                                                                          \
@@ -1707,14 +1758,15 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
                      records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, fillIndex, \
                      nIndex, fillB, nFillB, quads, outCoors, w.nRecords)
       // fixed kernel shapes: K1 threads per input; fill workgroups only for what there is to fill
-      const int64_t fillItems = (fillIndex ? nIndex : 0) + nFillB;
+      const int64_t fillItems = (probeFillIndex ? nIndex : 0) + nFillB;
       uint32_t planeFill = static_cast<uint32_t>((fillItems / 4 + kRbThreads - 1) / kRbThreads);
       if (planeFill > 1024) planeFill = 1024;
 #define D3D_LAUNCH_PROBE_PLANE(SUBM, K1, K2, K3)                                                                    \
   hipLaunchKernelGGL((bmProbePlane<SUBM, K1, K2, K3>), dim3(planeFill + probeBlocks * K1 + extra), block, 0, stream, \
                      g, m, coors, numActIn, cap, pitch, records, chunkBase, perm, permShuffled, maxNumActOut,     \
-                     staging, cnt, w.nBlocks, totals, fillIndex, nIndex, fillB, nFillB, planeFill, probeBlocks,     \
-                     outCoors, w.nRecords)
+                     staging, cnt, w.nBlocks, totals, probeFillIndex, nIndex, fillB, nFillB, planeFill,             \
+                     probeBlocks, outCoors, w.nRecords, probeMasks ? masks : nullptr, (skipIndex && subM) ? 1 : 0,   \
+                     directScatter ? nbrOut : nullptr, nbrRows)
       if (subM) {
         switch (ksel) {
           case 1: D3D_LAUNCH_PROBE_PLANE(true, 3, 3, 3); break;
@@ -1770,7 +1822,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
                        static_cast<int64_t>(g.kVol) * nbrRows);
   hipLaunchKernelGGL(rbCompact, perTap, block, 0, stream, numActIn, cap, pitch, g.kVol, staging, cnt, w.nBlocks,
                      totals, index, index + rowLen, index + 2 * rowLen, numIndex, nbrRows > 0 ? nbrOut : nullptr, nbrRows,
-                     compactPerm, compactPermFlag, mirror ? 1 : 0, inPlace ? 1 : 0, masks, fillState, incremental ? 1 : 0);
+                     compactPerm, compactPermFlag, mirror ? 1 : 0, inPlace ? 1 : 0, compactMasks, fillState,
+                     incremental ? 1 : 0, skipIndex ? 1 : 0);
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;
 }

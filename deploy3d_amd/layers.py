@@ -9,7 +9,7 @@ it can be captured into a HIP graph.
 import numpy as np
 import torch
 
-from .plugin import OPT_PERSISTENT_INDEX, Plugin, TensorDesc
+from .plugin import OPT_INDEX_UNUSED, OPT_PERSISTENT_INDEX, Plugin, TensorDesc
 from .spconv_index import index_blob
 from .spconv_mm import mm_blob
 
@@ -132,9 +132,13 @@ class SparseBackbone:
     stream waited for that rulebook (an event edge straight from one side stream to the other made
     hipStreamEndCapture crash in the runtime).  The side streams fork from and join into the caller's current
     stream, so a forward pass can still be captured into one HIP graph (it then holds parallel branches).
+
+    ``index_tensors=False`` tells the rulebook operators that nothing outside this runner reads their index tensors
+    (``Rulebook.index`` is then unspecified): they write the tables the convolutions read and skip the compaction.
     """
 
-    def __init__(self, layers, weights, capacities, dtype=torch.float16, device="cuda", overlap=True):
+    def __init__(self, layers, weights, capacities, dtype=torch.float16, device="cuda", overlap=True,
+                 index_tensors=True):
         self.specs = layers
         self.layers = [SparseConvLayer(s, w, b, cap, dtype=dtype, device=device)
                        for s, (w, b), cap in zip(layers, weights, capacities)]
@@ -143,6 +147,15 @@ class SparseBackbone:
         owner = {}
         for spec, lyr in zip(layers, self.layers):
             lyr.mm_plugin.link_rulebook(owner.setdefault(spec["key"], lyr).idx_plugin)
+        # index_tensors=False: this runner is the only reader of the index tensors and its convolutions read the
+        # linked tables, so the rulebook operators may leave the tensors unwritten (D3D_OPT_INDEX_UNUSED) - except
+        # for a key that an inverse convolution uses, which works from the tensor
+        if not index_tensors:
+            inverse_keys = {spec["key"] for spec in layers if spec.get("inverse", False)}
+            for key, lyr in owner.items():
+                if key not in inverse_keys:
+                    lyr.idx_plugin.set_option(OPT_INDEX_UNUSED, 1)
+        self.index_tensors = index_tensors
         self.overlap = overlap
         self._side = None
 

@@ -30,6 +30,7 @@ EXPORTS = [
     "d3d_enqueue_static", "d3d_link_rulebook", "d3d_link_coords", "d3d_set_option",
 ]
 OPT_PERSISTENT_INDEX = 1
+OPT_INDEX_UNUSED = 2
 
 
 class EngineError(RuntimeError):

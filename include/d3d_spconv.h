@@ -189,8 +189,15 @@ int32_t d3d_link_coords(d3d_plugin* subm, d3d_plugin* producer);
  * to -1 only the slots its previous pass used and the new one does not, instead of the whole tensor at capacity
  * (reference: cudaMemsetAsync of the whole tensor, trt/spconv/index.cu:352-354); after every enqueue the tensor
  * still reads -1 in every unused slot.  The first enqueue on a buffer, and the first after the buffer or its shape
- * changed, fill it whole. */
-enum { D3D_OPT_PERSISTENT_INDEX = 1 };
+ * changed, fill it whole.
+ * D3D_OPT_INDEX_UNUSED (SPConvIdx{N}d; value 0 / 1): the caller promises that nothing reads the index tensor
+ * (output 0) except forward convolutions linked to this operator with d3d_link_rulebook - the situation of an
+ * engine in which the tensor is an edge between these nodes only.  Where the operator can write what those
+ * convolutions read without compacting the pairs (3-D kernels 3x3x3, 3x1x1, 3x1x3, 1x3x3 at dilation 1 on the
+ * occupancy map), it then leaves output 0 unwritten: its content is unspecified, numIndex (output 1) and the
+ * coordinate outputs are written as always.  Without linked convolutions, and for every other geometry, the
+ * option changes nothing.  An inverse convolution, an unlinked one, or any other reader of output 0 needs it off. */
+enum { D3D_OPT_PERSISTENT_INDEX = 1, D3D_OPT_INDEX_UNUSED = 2 };
 int32_t d3d_set_option(d3d_plugin* p, int32_t option, int64_t value);
 
 #ifdef __cplusplus

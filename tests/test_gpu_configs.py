@@ -44,6 +44,53 @@ def compare_chain(cfg, net, ref, tol_scale=1.0):
             assert err <= 2e-2 * rms * tol_scale, (spec["name"], err, rms)
 
 
+@pytest.mark.parametrize("config,n", [(3, 12000), (5, 20000), (1, 5000), (2, 8000)])
+def test_unwritten_index_tensors_give_the_same_pass(engine, config, n):
+    """D3D_OPT_INDEX_UNUSED (index_tensors=False): the rulebook operators write tables and tile masks in the probe
+    pass and leave the index tensors unwritten.  Every layer's features, coordinates and live count must equal the
+    full pass bit for bit - with rows in rank order and shuffled (config 1 and the first stage of config 3 feed
+    unsorted voxels), with fewer live voxels in the same buffers, eager and under HIP-graph replay; numIndex is
+    still written."""
+    from deploy3d_amd import layers, synth
+    cfg = {1: synth.config1, 2: synth.config2, 3: synth.config3, 5: synth.config5}[config](n)
+    specs, weights = cfg["layers"], cfg["weights"]
+    n = len(cfg["coords"])
+    counts = layers.measure_output_counts(specs, cfg["coords"], cfg["grid"])
+    caps = layers.plan_capacities(specs, n, counts)
+    dtype = chain.TORCH_DTYPE[cfg["dtype"]]
+    full = layers.SparseBackbone(specs, weights, caps, dtype=dtype, overlap=False)
+    lean = layers.SparseBackbone(specs, weights, caps, dtype=dtype, overlap=False, index_tensors=False)
+    x = layers.make_input(cfg["coords"], cfg["feats"], cfg["grid"], dtype=dtype)
+
+    def same():
+        for spec in specs:
+            a, b = full.outputs[spec["name"]], lean.outputs[spec["name"]]
+            m = int(a.num_act.item())
+            assert m == int(b.num_act.item()), spec["name"]
+            assert torch.equal(a.coors[:m], b.coors[:m]), spec["name"]
+            assert torch.equal(a.feats, b.feats), spec["name"]
+        for key, rb in full.rulebooks.items():
+            assert int(rb.num_index.item()) == int(lean.rulebooks[key].num_index.item()), key
+
+    for live in (n, n // 3, n):
+        x.num_act.fill_(live)
+        full.forward(x)
+        lean.forward(x)
+        torch.cuda.synchronize()
+        same()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            y = lean.forward(x)
+        for _ in range(3):
+            y.feats.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            same()
+
+
 def test_down_up_chain_with_inverse_convolution(engine):
     """An encoder-decoder wiring through the layer runner: strided down (key d), SubM at the lower resolution, then
     the inverse convolution of key d back onto the input sites, then a SubM that shares the first layer's key.  The
