@@ -405,8 +405,10 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
 }
 
 // Configuration per layer shape, measured on the layers of a VoxelNet backbone (120k voxels): rows per wavefront
-// 16 * MT, wavefronts per workgroup.  64 x 64 and narrower tiles afford 8 wavefronts; 128 output channels double
-// the accumulators, so the wavefront tile halves.  Layers with few rows (the 128-channel stages: 47 000 rows are
+// 16 * MT, wavefronts per workgroup.  64 x 64 and narrower tiles afford 8 wavefronts (4 wavefronts of 128 rows,
+// which read half the weight fragments per MFMA, measured slower on a 64 -> 64 layer: 68 us against 58 - one
+// wavefront per SIMD has nobody to hide its waits); 128 output channels double the accumulators, so the wavefront
+// tile halves.  Layers with few rows (the 128-channel stages: 47 000 rows are
 // 186 tiles of 256 rows for 256 CUs) pick the workgroup size whose tile count loads the CUs most evenly: the
 // time of a layer that fits one round is that of ONE tile, so 248 tiles of 192 rows beat 186 of 256.
 template <class T, int CIN, int COUT>

@@ -1820,7 +1820,10 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   if (nbrOut && nbrRows > 0 && !nbrFilled)
     hipLaunchKernelGGL(rbFillMinusOne, fillGrid(static_cast<int64_t>(g.kVol) * nbrRows / 4 + 1), block, 0, stream, nbrOut,
                        static_cast<int64_t>(g.kVol) * nbrRows);
-  hipLaunchKernelGGL(rbCompact, perTap, block, 0, stream, numActIn, cap, pitch, g.kVol, staging, cnt, w.nBlocks,
+  // with the index tensor unwritten only a build that may have to turn ranks into rows needs the whole grid; the
+  // others launch the one workgroup that writes numIndex
+  const dim3 compactGrid = (skipIndex && !compactPerm) ? dim3(1, 1) : perTap;
+  hipLaunchKernelGGL(rbCompact, compactGrid, block, 0, stream, numActIn, cap, pitch, g.kVol, staging, cnt, w.nBlocks,
                      totals, index, index + rowLen, index + 2 * rowLen, numIndex, nbrRows > 0 ? nbrOut : nullptr, nbrRows,
                      compactPerm, compactPermFlag, mirror ? 1 : 0, inPlace ? 1 : 0, compactMasks, fillState,
                      incremental ? 1 : 0, skipIndex ? 1 : 0);

@@ -20,7 +20,7 @@ import struct
 
 import torch
 
-from .plugin import OPT_PERSISTENT_INDEX, EngineError, Plugin, TensorDesc
+from .plugin import OPT_INDEX_UNUSED, OPT_PERSISTENT_INDEX, EngineError, Plugin, TensorDesc
 
 # onnx.TensorProto.DataType
 FLOAT, INT8, INT32, FLOAT16, BFLOAT16 = 1, 3, 6, 10, 16
@@ -359,7 +359,25 @@ class GraphExecutor:
                         self.plugins[src[0]].name.startswith("SPConvIdx") and \
                         producer.get(n.inputs[4]) == (src[0], 1):
                     p.link_rulebook(self.plugins[src[0]])
+        # an index tensor that only linked forward convolutions read (not a graph output, no other consumer) need
+        # not be written at all
+        outputs = {v.name for v in model.outputs}
+        for i, n in enumerate(self.nodes):
+            p = self.plugins.get(i)
+            if p is None or not p.name.startswith("SPConvIdx") or n.outputs[0] in outputs:
+                continue
+            readers = [(j, m) for j, m in enumerate(self.nodes) if n.outputs[0] in m.inputs]
+            if readers and all(j in self.plugins and self.plugins[j].name == "SPConvMM" and len(m.inputs) >= 5 and
+                               m.inputs[3] == n.outputs[0] and m.inputs[4] == n.outputs[1] and
+                               not self._inverse(m) for j, m in readers):
+                p.set_option(OPT_INDEX_UNUSED, 1)
         self._bound = None
+
+    @staticmethod
+    def _inverse(node):
+        """The `inverse` byte of an SPConvMM attribute blob (trt/spconv/mm_trt.cu:27-37: 4 x int32, subM, inverse)."""
+        blob = node.attrs.get("data", b"")
+        return len(blob) > 17 and blob[17] != 0
 
     @staticmethod
     def _toposort(model):
