@@ -9,20 +9,26 @@
 // Differences in HOW, all deliberate:
 //  * no host read-back of numActIn (index_trt.cu:207-209): grids are sized on
 //    the static capacity and every kernel reads the live count on the device;
-//  * the coordinate hash is one 64-bit slot per entry (key<<32 | value) in
-//    HBM, claimed with a single 64-bit CAS, so a probe is one 8-byte load;
-//  * every pass runs one workgroup per (chunk of 1024 inputs, tap), so all
-//    kVol*N probes or inserts of a pass are independent and in flight together;
+//  * two occupancy structures.  The default is a dense map of 64-cell bricks of the output grid (second half of
+//    this file): voxels are ranked in brick-major order by popcounts and a prefix over the bricks, a probe is a
+//    handful of neighbouring 16-byte records, strided outputs need no election and come out sorted.  Grids too
+//    large or too sparse for it take the coordinate hash (first half): one 64-bit slot per entry (key<<32 | value)
+//    in HBM, claimed with a single 64-bit CAS, so a probe is one 8-byte load;
+//  * the per-pair passes run one workgroup per (chunk of 1024 inputs, tap), so all kVol*N probes or inserts of a
+//    pass are independent and in flight together;
 //  * compaction is a prefix inside the workgroup plus per-(tap, chunk) counts;
 //    each workgroup sums the counts of its predecessors itself, so there are
 //    no device-wide scan kernels;
-//  * a strided output belongs to the contributing pair with the smallest
+//  * hash path: a strided output belongs to the contributing pair with the smallest
 //    (input row, tap) code (atomicMin) and outputs are numbered in (tap, input
 //    row) order of their owners, which makes the output order deterministic
-//    (the reference numbers them by hash-slot order, which depends on CAS races);
-//  * the strided hash is sized by the real bound on distinct outputs per input
+//    (the reference numbers them by hash-slot order, which depends on CAS races); the
+//    strided hash is sized by the real bound on distinct outputs per input
 //    (product over dims of the largest number of stride-compatible taps), not
-//    by 2*kVol*N slots.
+//    by 2*kVol*N slots;
+//  * besides the index tensor a build can write what the convolutions read - the pairs in output-major form and
+//    the tap masks of 64-row tiles (RbSide) - and can reuse the index tensor and the occupancy map of an earlier
+//    build (incremental fill, shared map).
 #include <cstdlib>
 #include <cstring>
 
