@@ -1280,7 +1280,7 @@ bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
   // tensor nobody reads needs no compaction: maskOut (SubM, staging rows = rows of the mirrored table) takes the
   // tile masks - a wavefront's 64 inputs are one 64-row tile - and fixTail has the rows between the live count
   // and the capacity set to -1; nbrDirect (strided) takes the pairs straight into the scattered table
-  // nbrDirect[tap][output row] = input row, filled with -1 by the reset pass, and nothing is staged.
+  // nbrDirect[tap][output row] = input row, filled with -1 by the reset pass; staging may then be null.
   constexpr int KP = K2 * K3;
   __shared__ uint4 group[4 * kRbThreads];
   __shared__ uint32_t ldsCnt[KP];
@@ -1386,12 +1386,9 @@ bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
         }
       }
       const int tap = (i1 * K2 + q2) * K3 + q3;
-      if (nbrDirect) {
-        if (row != kNone && row < static_cast<uint64_t>(nbrRows))
-          nbrDirect[static_cast<int64_t>(tap) * nbrRows + row] = static_cast<int32_t>(i);
-      } else if (inRange) {
-        staging[static_cast<int64_t>(tap) * pitch + i] = row;
-      }
+      if (nbrDirect && row != kNone && row < static_cast<uint64_t>(nbrRows))
+        nbrDirect[static_cast<int64_t>(tap) * nbrRows + row] = static_cast<int32_t>(i);
+      if (staging && inRange) staging[static_cast<int64_t>(tap) * pitch + i] = row;
       const uint32_t hits = static_cast<uint32_t>(__popcll(__ballot(row != kNone)));
       if (lane == q2 * K3 + q3) mine += hits;
       if (hits) tileBits |= 1ull << ((g.kVol - 1 - tap) & 63);
@@ -1678,6 +1675,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   side.masksWritten = masks != nullptr;
   bool nbrFilled = mirror;
   bool skipIndex = false;                     // set below when side.skipIndex can be honoured
+  bool directScatter = false;                 // the probe pass writes the scattered table itself
   unsigned long long* compactMasks = masks;   // null when the probe pass writes the masks itself
   const uint32_t* compactPerm = nullptr;      // block-map SubM: staging holds ranks, rows = perm[rank] when shuffled
   const uint32_t* compactPermFlag = nullptr;
@@ -1707,7 +1705,9 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     // place, or a strided build with a table to scatter into (which the reset pass then fills with -1, since the
     // probe pass writes entries into it).
     skipIndex = side.skipIndex && near && ksel != 0 && nbrOut && (subM ? (mirror && inPlace) : true);
-    const bool directScatter = skipIndex && !subM;
+    // (with the index tensor written it does not pay: the fill, moved into the reset pass, is no longer hidden
+    // beside the probe - measured 1-2 us slower per strided build)
+    directScatter = skipIndex && !subM;
     const bool probeMasks = subM && mirror && masks && near && ksel != 0;
     if (probeMasks) compactMasks = nullptr;
     side.indexWritten = !skipIndex;
@@ -1770,7 +1770,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
 #define D3D_LAUNCH_PROBE_PLANE(SUBM, K1, K2, K3)                                                                    \
   hipLaunchKernelGGL((bmProbePlane<SUBM, K1, K2, K3>), dim3(planeFill + probeBlocks * K1 + extra), block, 0, stream, \
                      g, m, coors, numActIn, cap, pitch, records, chunkBase, perm, permShuffled, maxNumActOut,     \
-                     staging, cnt, w.nBlocks, totals, probeFillIndex, nIndex, fillB, nFillB, planeFill,             \
+                     (directScatter && skipIndex) ? nullptr : staging, cnt, w.nBlocks, totals, probeFillIndex,      \
+                     nIndex, fillB, nFillB, planeFill,                                                               \
                      probeBlocks, outCoors, w.nRecords, probeMasks ? masks : nullptr, (skipIndex && subM) ? 1 : 0,   \
                      directScatter ? nbrOut : nullptr, nbrRows)
       if (subM) {
@@ -1830,7 +1831,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   // others launch the one workgroup that writes numIndex
   const dim3 compactGrid = (skipIndex && !compactPerm) ? dim3(1, 1) : perTap;
   hipLaunchKernelGGL(rbCompact, compactGrid, block, 0, stream, numActIn, cap, pitch, g.kVol, staging, cnt, w.nBlocks,
-                     totals, index, index + rowLen, index + 2 * rowLen, numIndex, nbrRows > 0 ? nbrOut : nullptr, nbrRows,
+                     totals, index, index + rowLen, index + 2 * rowLen, numIndex,
+                     (nbrRows > 0 && !directScatter) ? nbrOut : nullptr, nbrRows,
                      compactPerm, compactPermFlag, mirror ? 1 : 0, inPlace ? 1 : 0, compactMasks, fillState,
                      incremental ? 1 : 0, skipIndex ? 1 : 0);
   D3D_HIP_CHECK(hipGetLastError());
