@@ -297,6 +297,7 @@ def main():
         torch.cuda.synchronize()
         eager_ms = (time.perf_counter() - t0) * 1e3 / k_eager
         streams = "" if args.no_overlap else ", rulebooks beside convolutions on two side streams"
+        host_ms = None
         if args.no_graph:
             ms = eager_ms
             mode = "eager" + streams
@@ -311,6 +312,7 @@ def main():
             t0 = time.perf_counter()
             for _ in range(args.steps):
                 graph.replay()
+            host_ms = (time.perf_counter() - t0) * 1e3 / args.steps   # host time of one hipGraphLaunch
             torch.cuda.synchronize()
             ms = (time.perf_counter() - t0) * 1e3 / args.steps
             mode = "hip-graph replay" + streams
@@ -426,6 +428,7 @@ def main():
         "effective_tflops": round(total_flops / (ms * 1e-3) / 1e12, 2),
         "total_gflop": round(total_flops / 1e9, 2),
         "eager_ms_per_step": round(eager_ms, 4),
+        "host_ms_per_graph_launch": None if host_ms is None else round(host_ms, 4),
         "outputs_match_warmup": same,
         "layer_ms": {s["name"]: round(t, 4) for s, t in zip(specs, layer_ms)},
         "rulebook_ms": {k: round(t, 4) for k, t in rulebook_ms.items()},
