@@ -408,7 +408,10 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
 // 16 * MT, wavefronts per workgroup.  64 x 64 and narrower tiles afford 8 wavefronts (4 wavefronts of 128 rows,
 // which read half the weight fragments per MFMA, measured slower on a 64 -> 64 layer: 68 us against 58 - one
 // wavefront per SIMD has nobody to hide its waits); 128 output channels double the accumulators, so the wavefront
-// tile halves.  Layers with few rows (the 128-channel stages: 47 000 rows are
+// tile halves.  32 -> 32 takes 8 wavefronts as well (two workgroups of 78 KB per CU, 16 wavefronts): 38 us against
+// 41 with 4, 40 with three 4-wavefront workgroups per CU, 41 with 128-row wavefront tiles; with gathers and MFMAs
+// both taken out of it the kernel still runs 27 us on that layer (25 with the table reads served from cache), so
+// what is left is the per-step bookkeeping of a 32-channel step, not a memory or matrix limit.  Layers with few rows (the 128-channel stages: 47 000 rows are
 // 186 tiles of 256 rows for 256 CUs) pick the workgroup size whose tile count loads the CUs most evenly: the
 // time of a layer that fits one round is that of ONE tile, so 248 tiles of 192 rows beat 186 of 256.
 template <class T, int CIN, int COUT>
@@ -429,6 +432,8 @@ int32_t launchPipeShape(const ConvArgs& a, hipStream_t stream) {
     if (best == 6) return launchPipeCfg<T, CIN, COUT, 2, 6>(a, stream);
     if (best == 4) return launchPipeCfg<T, CIN, COUT, 2, 4>(a, stream);
     return launchPipeCfg<T, CIN, COUT, 2, 8>(a, stream);
+  } else if constexpr (CIN == 32 && COUT == 32) {
+    return launchPipeCfg<T, CIN, COUT, 4, 8>(a, stream);
   } else {
     return launchPipeCfg<T, CIN, COUT, 4, 4>(a, stream);
   }

@@ -805,20 +805,41 @@ bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, u
        uint32_t* groupTickets, int32_t* numActOut, int32_t maxNumActOut) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   __shared__ uint32_t isLast;
-  const uint32_t first = blockIdx.x * kRbChunk + threadIdx.x * kRbItems;
+  // A wavefront takes 256 consecutive records as 4 rows of 64: lane l reads records l, 64 + l, 128 + l, 192 + l of
+  // them, so every load instruction covers 1 KB of consecutive memory.  Counts are at most 64 and a row's running
+  // sum at most 4096, so two rows share one 32-bit lane scan (16 bits each).
+  static_assert(kRbItems == 4 && kRbChunk == 4 * 256, "bmScan assumes 4 wavefronts of 4 x 64 records");
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t first = blockIdx.x * kRbChunk + wave * 256 + lane;
   uint32_t count[kRbItems];
-  uint32_t mine = 0;
 #pragma unroll
-  for (int j = 0; j < kRbItems; ++j) {
-    count[j] = first + j < nRecords ? static_cast<uint32_t>(__popcll(records[first + j].bits)) : 0u;
-    mine += count[j];
+  for (int j = 0; j < kRbItems; ++j)
+    count[j] = first + j * 64 < nRecords ? static_cast<uint32_t>(__popcll(records[first + j * 64].bits)) : 0u;
+  uint32_t inclA = count[0] | (count[1] << 16), inclB = count[2] | (count[3] << 16);
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t upA = __shfl_up(inclA, off, 64), upB = __shfl_up(inclB, off, 64);
+    if (lane >= off) {
+      inclA += upA;
+      inclB += upB;
+    }
   }
-  uint32_t total;
-  uint32_t rank = blockExclusiveScan(mine, scratch, &total);
+  const uint32_t endA = __shfl(inclA, 63, 64), endB = __shfl(inclB, 63, 64);
+  const uint32_t rowSum[kRbItems] = {endA & 0xFFFFu, endA >> 16, endB & 0xFFFFu, endB >> 16};
+  const uint32_t incl[kRbItems] = {inclA & 0xFFFFu, inclA >> 16, inclB & 0xFFFFu, inclB >> 16};
+  if (lane == 0) scratch[wave] = rowSum[0] + rowSum[1] + rowSum[2] + rowSum[3];
+  __syncthreads();
+  uint32_t rank = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < kRbThreads / 64; ++w) {
+    if (w < wave) rank += scratch[w];
+    total += scratch[w];
+  }
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
-    if (count[j]) records[first + j].prefix = rank;  // an empty record is never ranked: on sparse grids most are
-    rank += count[j];
+    // an empty record is never ranked: on sparse grids most are
+    if (count[j]) records[first + j * 64].prefix = rank + incl[j] - count[j];
+    rank += rowSum[j];
   }
   if (threadIdx.x == 0) {
     // The chunk totals are the only data that passes between workgroups inside this kernel, and every access to
