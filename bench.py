@@ -346,6 +346,26 @@ def main():
                      "outputs_equal_full_pass": bool(n2 == int(y.num_act.item()) and torch.equal(y2.feats, y.feats)
                                                      and torch.equal(y2.coors[:n2], y.coors[:n2]))}
             del net2, graph2
+        # third figure: the same pass recorded once as a native schedule (d3d_schedule_*, three lanes with direct
+        # events, no HIP graph) - what a caller without graph capture gets; its host cost per pass is reported
+        sched = None
+        if not args.no_graph and not args.no_fused and all("+" not in (s.get("src") or "") for s in specs):
+            net3 = layers.SparseBackbone(specs, weights, caps, dtype=dtype, overlap=False)
+            for _ in range(3):
+                y3 = net3.forward_scheduled(x)
+            stream.synchronize()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                net3.forward_scheduled(x)
+            host3 = (time.perf_counter() - t0) * 1e3 / args.steps
+            torch.cuda.synchronize()
+            ms3 = (time.perf_counter() - t0) * 1e3 / args.steps
+            sched = {"ms_per_step": round(ms3, 4), "host_ms_per_pass": round(host3, 4),
+                     "what": "the pass enqueued by one d3d_schedule_run per step: no HIP graph, rulebooks on two "
+                             "lanes of their own, events straight between the lanes",
+                     "outputs_equal_full_pass": bool(torch.equal(y3.feats, y.feats))}
+            del net3
         n_final = int(y.num_act.item())
         gpu_coords = y.coors[:n_final].cpu().numpy()
         gpu_feats = y.feats[:n_final].float().cpu().numpy() if dtype != torch.int8 else y.feats[:n_final].cpu().numpy()
@@ -433,6 +453,7 @@ def main():
         "layer_ms": {s["name"]: round(t, 4) for s, t in zip(specs, layer_ms)},
         "rulebook_ms": {k: round(t, 4) for k, t in rulebook_ms.items()},
         "index_unused": fused,
+        "native_schedule": sched,
         "roofline": roofline,
         "rooflines": rooflines,
         "measured_peak": peaks,

@@ -9,7 +9,7 @@ it can be captured into a HIP graph.
 import numpy as np
 import torch
 
-from .plugin import OPT_INDEX_UNUSED, OPT_PERSISTENT_INDEX, Plugin, TensorDesc
+from .plugin import OPT_INDEX_UNUSED, OPT_PERSISTENT_INDEX, Plugin, Schedule, TensorDesc
 from .spconv_index import index_blob
 from .spconv_mm import mm_blob
 
@@ -209,6 +209,45 @@ class SparseBackbone:
         self.inputs = inputs    # layer name -> the SparseTensor it read
         self.outputs = outs
         return cur
+
+
+    # -- the pass as one native call -------------------------------------------------------------------------
+    def build_schedule(self, x):
+        """Records the pass on ``x`` as a native schedule (d3d_schedule_*): convolutions on lane 0 (the caller's
+        stream), strided rulebooks on lane 1, SubM rulebooks on lane 2; a convolution waits for its rulebook, a SubM
+        rulebook for the strided rulebook that wrote its coordinates (directly - no detour through the main
+        stream, which only stream capture needs).  Runs one ordinary pass first so that every buffer exists."""
+        if any("+" in (spec.get("src") or "") for spec in self.specs):
+            raise NotImplementedError("a schedule holds operator steps only; this chain adds feature maps in between")
+        self.forward(x)
+        sched = Schedule(lanes=3)
+        rb_step, by_plugin = {}, {}
+        for spec, lyr in zip(self.specs, self.layers):
+            inp = self.inputs[spec["name"]]
+            key = spec["key"]
+            rb = self.rulebooks[key]
+            if key not in rb_step:
+                st = lyr._idx_state
+                after = [by_plugin[id(inp.producer)]] if inp.producer is not None and id(inp.producer) in by_plugin else []
+                rb_step[key] = sched.add(lyr.idx_plugin, st["in_descs"], st["out_descs"], [inp.coors, inp.num_act, None],
+                                         st["outs"], st["ws"], lane=2 if spec["subm"] else 1, after=after)
+                by_plugin[id(lyr.idx_plugin)] = rb_step[key]
+            inverse = bool(spec.get("inverse", False))
+            num_in, num_out = (rb.num_act_out, rb.num_act_in) if inverse else (rb.num_act_in, rb.num_act_out)
+            st = lyr._mm_state
+            sched.add(lyr.mm_plugin, st["in_descs"], st["out_descs"], [inp.feats, num_in, num_out, rb.index, rb.num_index],
+                      [st["out"]], None, lane=0, after=[rb_step[key]])
+        self._schedule = (sched, (x.feats.data_ptr(), x.coors.data_ptr(), x.num_act.data_ptr()))
+        return sched
+
+    def forward_scheduled(self, x):
+        """The pass through the native schedule (recorded at the first call, and again when ``x`` is another set of
+        buffers); same output tensors as ``forward``."""
+        sig = (x.feats.data_ptr(), x.coors.data_ptr(), x.num_act.data_ptr())
+        if getattr(self, "_schedule", None) is None or self._schedule[1] != sig:
+            self.build_schedule(x)
+        self._schedule[0].run()
+        return self.outputs[self.specs[-1]["name"]]
 
 
 def plan_capacities(layers, n_in, counts=None):

@@ -20,7 +20,7 @@ import struct
 
 import torch
 
-from .plugin import OPT_INDEX_UNUSED, OPT_PERSISTENT_INDEX, EngineError, Plugin, TensorDesc
+from .plugin import OPT_INDEX_UNUSED, OPT_PERSISTENT_INDEX, EngineError, Plugin, Schedule, TensorDesc
 
 # onnx.TensorProto.DataType
 FLOAT, INT8, INT32, FLOAT16, BFLOAT16 = 1, 3, 6, 10, 16
@@ -433,6 +433,32 @@ class GraphExecutor:
             else:
                 _, p, in_descs, out_descs, ins, outs, ws = step
                 p.enqueue(in_descs, out_descs, ins, outs, ws)
+        return {v.name: self._bound["values"][v.name] for v in self.model.outputs}
+
+
+    def run_scheduled(self, **inputs):
+        """``run`` through a native schedule (d3d_schedule_*): every node becomes a step that waits for the steps
+        its inputs come from; rulebook nodes get lanes of their own (strided 1, SubM 2), everything else runs on
+        the current stream.  Graphs of plugin nodes only (an ``Add`` needs the step-by-step ``run``)."""
+        sig = {k: (tuple(v.shape), v.dtype, v.data_ptr()) for k, v in inputs.items()}
+        if self._bound is None or self._bound["shapes"] != sig:
+            self.run(**inputs)  # binds, and brings every operator's buffers into being
+        if "schedule" not in self._bound:
+            if any(step[0] != "plugin" for step in self._bound["plan"]):
+                raise NotImplementedError("a schedule holds plugin steps only")
+            sched = Schedule(lanes=3)
+            made = {}  # tensor name -> step that writes it
+            plugin_nodes = [n for n in self.nodes if n.op_type == "TRT_PluginV2"]
+            for n, (_, p, in_descs, out_descs, ins, outs, ws) in zip(plugin_nodes, self._bound["plan"]):
+                lane = 0
+                if p.name.startswith("SPConvIdx"):
+                    lane = 2 if len(n.attrs["data"]) >= 2 and n.attrs["data"][-2] != 0 else 1   # the subM byte
+                after = sorted({made[name] for name in n.inputs if name in made})
+                step = sched.add(p, in_descs, out_descs, ins, outs, ws, lane=lane, after=after)
+                for name in n.outputs:
+                    made[name] = step
+            self._bound["schedule"] = sched
+        self._bound["schedule"].run()
         return {v.name: self._bound["values"][v.name] for v in self.model.outputs}
 
 

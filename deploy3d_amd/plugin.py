@@ -28,6 +28,7 @@ EXPORTS = [
     "d3d_serialize", "d3d_num_outputs", "d3d_output_dims", "d3d_output_dtype", "d3d_supports_format",
     "d3d_configure", "d3d_workspace_size", "d3d_enqueue", "d3d_last_error", "d3d_num_ops", "d3d_op_name",
     "d3d_enqueue_static", "d3d_link_rulebook", "d3d_link_coords", "d3d_set_option",
+    "d3d_schedule_create", "d3d_schedule_add", "d3d_schedule_size", "d3d_schedule_run", "d3d_schedule_destroy",
 ]
 OPT_PERSISTENT_INDEX = 1
 OPT_INDEX_UNUSED = 2
@@ -116,6 +117,17 @@ def load_library(path=None):
     lib.d3d_link_coords.argtypes = [vp, vp]
     lib.d3d_set_option.restype = i32
     lib.d3d_set_option.argtypes = [vp, i32, ctypes.c_int64]
+    lib.d3d_schedule_create.restype = i32
+    lib.d3d_schedule_create.argtypes = [i32, ctypes.POINTER(vp)]
+    lib.d3d_schedule_add.restype = i32
+    lib.d3d_schedule_add.argtypes = [vp, vp, descp, i32, descp, i32, ctypes.POINTER(vp), ctypes.POINTER(vp), vp, sz,
+                                     i32, ctypes.POINTER(i32), i32]
+    lib.d3d_schedule_size.restype = i32
+    lib.d3d_schedule_size.argtypes = [vp]
+    lib.d3d_schedule_run.restype = i32
+    lib.d3d_schedule_run.argtypes = [vp, vp]
+    lib.d3d_schedule_destroy.restype = None
+    lib.d3d_schedule_destroy.argtypes = [vp]
     _lib = lib
     return lib
 
@@ -234,6 +246,51 @@ class Plugin:
             return
         _check(self._lib.d3d_enqueue(self._h, _desc_array(in_descs), _desc_array(out_descs), ptrs(inputs),
                                      ptrs(outputs), ws_ptr, ws_bytes, ctypes.c_void_p(stream)))
+
+
+class Schedule:
+    """A pass recorded once and enqueued by one native call (d3d_schedule_*): steps are operator enqueues with their
+    descriptors, tensors and workspace, each on a lane (lane 0 = the stream of ``run``; the others are streams the
+    schedule owns) and behind the earlier steps it names.  Keeps the tensors and operators it was given alive."""
+
+    def __init__(self, lanes=1):
+        self._lib = load_library()
+        h = ctypes.c_void_p()
+        _check(self._lib.d3d_schedule_create(int(lanes), ctypes.byref(h)))
+        self._h = h
+        self.lanes = int(lanes)
+        self._keep = []
+
+    def add(self, plugin, in_descs, out_descs, inputs, outputs, workspace=None, lane=0, after=()):
+        """Appends ``plugin.enqueue(in_descs, out_descs, inputs, outputs, workspace)``; returns the step's index."""
+        def ptrs(ts):
+            arr = (ctypes.c_void_p * max(1, len(ts)))()
+            for i, t in enumerate(ts):
+                arr[i] = None if t is None or t.numel() == 0 else t.data_ptr()
+            return arr
+        ws_ptr = None if workspace is None else workspace.data_ptr()
+        ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+        dep = (ctypes.c_int32 * max(1, len(after)))(*[int(a) for a in after])
+        rc = self._lib.d3d_schedule_add(self._h, plugin._h, _desc_array(in_descs), len(in_descs),
+                                        _desc_array(out_descs), len(out_descs), ptrs(inputs), ptrs(outputs), ws_ptr,
+                                        ws_bytes, int(lane), dep, len(after))
+        if rc < 0:
+            _check(rc)
+        self._keep.append((plugin, list(inputs), list(outputs), workspace))
+        return rc
+
+    def __len__(self):
+        return int(self._lib.d3d_schedule_size(self._h))
+
+    def run(self, stream=None):
+        if stream is None:
+            stream = torch.cuda.current_stream().cuda_stream
+        _check(self._lib.d3d_schedule_run(self._h, ctypes.c_void_p(stream)))
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.d3d_schedule_destroy(h)
 
 
 STATIC_SCRATCH_BYTES = 64 << 20

@@ -200,6 +200,35 @@ int32_t d3d_link_coords(d3d_plugin* subm, d3d_plugin* producer);
 enum { D3D_OPT_PERSISTENT_INDEX = 1, D3D_OPT_INDEX_UNUSED = 2 };
 int32_t d3d_set_option(d3d_plugin* p, int32_t option, int64_t value);
 
+/* ---- a pass as one native call -------------------------------------------------------------------------------
+ * Replaces, for a chain of these operators, what TensorRT's execution context does in the reference
+ * (IExecutionContext::enqueueV3 walking the engine's layers; the reference drives it from
+ * deploy3d/symfun/trt_utils/trt_onnx_module.py:186-250): the caller describes the pass once, step by step, and a run
+ * then enqueues every step from native code, on several HIP streams where the steps allow it.
+ *
+ * d3d_schedule_create: `n_lanes` streams (1..8).  Lane 0 is the stream handed to d3d_schedule_run; the others are
+ *   streams the schedule creates (default priority) and owns.
+ * d3d_schedule_add: appends one d3d_enqueue call - operator, descriptors, device pointers, workspace - to run on
+ *   `lane`, after the earlier steps listed in `after` (their return values).  Steps of one lane run in the order
+ *   added.  Descriptors and pointer arrays are copied; the operator, the tensors and the workspace must outlive the
+ *   schedule's runs, and the operator must be configured as for d3d_enqueue.  Returns the step's index (>= 0) or a
+ *   negative status.
+ * d3d_schedule_run: enqueues all steps; the owned lanes start behind what `stream` holds at the call and `stream`
+ *   continues behind all of them, so for the caller the run is stream-ordered work on `stream`.  No host
+ *   synchronisation.  Returns the first failing status; steps behind a failed one are not enqueued.  Refused with
+ *   D3D_ERR_UNSUPPORTED while `stream` is capturing (capture the operators' own enqueues instead).  One thread at
+ *   a time per schedule.
+ * d3d_schedule_destroy: waits for the owned lanes, then frees them; the operators stay the caller's. */
+typedef struct d3d_schedule d3d_schedule;
+int32_t d3d_schedule_create(int32_t n_lanes, d3d_schedule** out);
+int32_t d3d_schedule_add(d3d_schedule* s, d3d_plugin* plugin, const d3d_tensor_desc* in_desc, int32_t nb_in,
+                         const d3d_tensor_desc* out_desc, int32_t nb_out, const void* const* inputs,
+                         void* const* outputs, void* workspace, size_t workspace_bytes, int32_t lane,
+                         const int32_t* after, int32_t nb_after);
+int32_t d3d_schedule_size(const d3d_schedule* s);
+int32_t d3d_schedule_run(d3d_schedule* s, void* stream);
+void d3d_schedule_destroy(d3d_schedule* s);
+
 #ifdef __cplusplus
 }
 #endif

@@ -214,3 +214,33 @@ def test_short_workspace_is_refused_before_any_launch():
     need = p.workspace_size(ins, outs)
     bufs = [torch.zeros(d.shape(), dtype=torch.float32 if i == 0 else torch.int32) for i, d in enumerate(outs)]
     assert enqueue(p, ins, outs, [pts, bidx, conf, None], bufs, need - 1).status == -5
+
+
+def test_schedule_bookkeeping_without_a_gpu():
+    """d3d_schedule_*: a one-lane schedule needs no HIP object, so its bookkeeping is testable here - step indices,
+    refused steps (wrong output count, a wait for a step that does not precede, a lane outside the schedule)."""
+    from deploy3d_amd.plugin import Schedule
+    lib = deploy3d_amd.load_library()
+    h = ctypes.c_void_p()
+    assert lib.d3d_schedule_create(0, ctypes.byref(h)) == -3 and lib.d3d_schedule_create(9, ctypes.byref(h)) == -3
+    assert lib.d3d_schedule_size(None) == -3 and lib.d3d_schedule_run(None, None) == -3
+    lib.d3d_schedule_destroy(None)
+    p = Plugin("SPConvIdx3d", index_blob((3,) * 3, (1,) * 3, (1,) * 3, (1,) * 3, (0,) * 3, 64, True, False))
+    ins = [TensorDesc.of((64, 4), torch.int32), TensorDesc.of((1,), torch.int32),
+           TensorDesc.of((1, 0, 8, 8, 8), torch.int32)]
+    outs = p.output_descs(ins)
+    coors, num = torch.zeros((64, 4), dtype=torch.int32), torch.zeros(1, dtype=torch.int32)
+    index, num_index = torch.empty(outs[0].shape(), dtype=torch.int32), torch.zeros(1, dtype=torch.int32)
+    s = Schedule(lanes=1)
+    assert len(s) == 0
+    assert s.add(p, ins, outs, [coors, num, None], [index, num_index]) == 0
+    assert s.add(p, ins, outs, [coors, num, None], [index, num_index], after=[0]) == 1
+    assert len(s) == 2
+    with pytest.raises(EngineError) as e:
+        s.add(p, ins, outs[:1], [coors, num, None], [index])           # the operator has two outputs
+    assert e.value.status == -3
+    with pytest.raises(EngineError):
+        s.add(p, ins, outs, [coors, num, None], [index, num_index], after=[2])   # itself
+    with pytest.raises(EngineError):
+        s.add(p, ins, outs, [coors, num, None], [index, num_index], lane=1)
+    assert len(s) == 2

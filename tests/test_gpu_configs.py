@@ -91,6 +91,45 @@ def test_unwritten_index_tensors_give_the_same_pass(engine, config, n):
             same()
 
 
+@pytest.mark.parametrize("config,n,index_tensors", [(3, 12000, True), (3, 12000, False), (2, 20000, True)])
+def test_native_schedule_equals_the_stream_runner(engine, config, n, index_tensors):
+    """d3d_schedule_*: the pass recorded once and enqueued by one native call on three lanes gives, bit for bit,
+    the features, coordinates and index tensors of the same runner enqueuing operator by operator - over passes of
+    different live counts - and refuses to run on a capturing stream."""
+    from deploy3d_amd import EngineError, layers, synth
+    cfg = (synth.config3 if config == 3 else synth.config2)(n)
+    specs, weights = cfg["layers"], cfg["weights"]
+    n = len(cfg["coords"])
+    counts = layers.measure_output_counts(specs, cfg["coords"], cfg["grid"])
+    caps = layers.plan_capacities(specs, n, counts)
+    plain = layers.SparseBackbone(specs, weights, caps, overlap=False, index_tensors=index_tensors)
+    sched = layers.SparseBackbone(specs, weights, caps, overlap=False, index_tensors=index_tensors)
+    x = layers.make_input(cfg["coords"], cfg["feats"], cfg["grid"])
+    for live in (n, n // 3, n):
+        x.num_act.fill_(live)
+        plain.forward(x)
+        y = sched.forward_scheduled(x)
+        torch.cuda.synchronize()
+        assert len(sched._schedule[0]) == len(specs) + len(sched.rulebooks)
+        assert y is sched.outputs[specs[-1]["name"]]
+        for spec in specs:
+            a, b = plain.outputs[spec["name"]], sched.outputs[spec["name"]]
+            k = int(a.num_act.item())
+            assert k == int(b.num_act.item()), spec["name"]
+            assert torch.equal(a.feats, b.feats) and torch.equal(a.coors[:k], b.coors[:k]), spec["name"]
+        if index_tensors:
+            for key, rb in plain.rulebooks.items():
+                assert torch.equal(rb.index, sched.rulebooks[key].index), key
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            x.num_act.fill_(n)
+            with pytest.raises(EngineError) as e:
+                sched._schedule[0].run()
+    assert e.value.status == -1
+
+
 def test_down_up_chain_with_inverse_convolution(engine):
     """An encoder-decoder wiring through the layer runner: strided down (key d), SubM at the lower resolution, then
     the inverse convolution of key d back onto the input sites, then a SubM that shares the first layer's key.  The

@@ -63,6 +63,22 @@ def test_whole_configurations_and_graph_capture(engine, config, n):
         torch.cuda.synchronize()
         _same(y, out, ex.model)
         assert torch.equal(out["bev"], bev)
+    # the same graph through the native schedule: one call per pass, rulebook nodes on lanes of their own
+    if config == 3:
+        for live in (n // 3, n):
+            x.num_act.fill_(live)
+            y = net.forward(x)
+            bev = layers.densify(y)
+            for name in ("bev", ex.model.outputs[0].name):
+                ex._bound["values"][name].zero_()
+            out = ex.run_scheduled(**_graph_inputs(x, cfg["grid"]))
+            torch.cuda.synchronize()
+            _same(y, out, ex.model)
+            assert torch.equal(out["bev"], bev)
+        assert len(ex._bound["schedule"]) == len(ex.nodes)
+    else:
+        with pytest.raises(NotImplementedError):
+            ex.run_scheduled(**_graph_inputs(x, cfg["grid"]))
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         inputs = _graph_inputs(x, cfg["grid"])
