@@ -187,6 +187,33 @@ __device__ __forceinline__ uint32_t blockExclusiveScan(uint32_t v, uint32_t* scr
   return waveBase + incl - v;
 }
 
+// Both at once behind one pair of barriers: *sum gets the workgroup sum of `a`, the return value is the exclusive
+// prefix of `v` in thread order.  scratch: 2 * kRbThreads / 64 words.
+__device__ __forceinline__ uint32_t blockSumAndScan(uint32_t a, uint32_t v, uint32_t* scratch, uint32_t* sum) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  uint32_t incl = v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += up;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) a += __shfl_down(a, off, 64);
+  __syncthreads();
+  if (lane == 63) scratch[wave] = incl;
+  if (lane == 0) scratch[kRbThreads / 64 + wave] = a;
+  __syncthreads();
+  uint32_t waveBase = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < kRbThreads / 64; ++w) {
+    if (w < wave) waveBase += scratch[w];
+    total += scratch[kRbThreads / 64 + w];
+  }
+  *sum = total;
+  return waveBase + incl - v;
+}
+
 // ---------------------------------------------------------------------------
 // reset: hash slots = EMPTY, index tensor = -1, tap totals = 0.  One streaming
 // pass of 16-byte stores (replaces resetHashKernel + the cudaMemsetAsync calls
@@ -497,14 +524,17 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
           int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* nbr, int64_t nbrRows,
           const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int mirror, int inPlace,
           unsigned long long* __restrict__ masks, uint32_t* fillState, int incrementalFill, int skipIndex) {
-  __shared__ uint32_t scratch[kRbThreads / 64];
+  __shared__ uint32_t scratch[2 * kRbThreads / 64];
   const int tap = blockIdx.y;
   const uint32_t b = blockIdx.x;
-  if (b == 0 && tap == 0 && threadIdx.x == 0) {
-    uint32_t end = 0;
-    for (int t = 0; t < kVol; ++t) end += tapSegment(totals, t);
-    *numIndex = static_cast<int32_t>(end);
-    if (fillState) fillState[1] = end;  // what this pass uses of the index tensor: the next pass clears from here
+  if (b == 0 && tap == 0) {  // workgroup-uniform
+    uint32_t part = 0;
+    for (int t = threadIdx.x; t < kVol; t += blockDim.x) part += tapSegment(totals, t);
+    const uint32_t end = blockSum(part, scratch);
+    if (threadIdx.x == 0) {
+      *numIndex = static_cast<int32_t>(end);
+      if (fillState) fillState[1] = end;  // what this pass uses of the index tensor: the next pass clears from here
+    }
   }
   if (skipIndex) {
     // Nobody reads the index tensor and the probe pass has written table and masks: what is left is turning ranks
@@ -528,11 +558,14 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
   // behind the new end is short unless the scene changed a lot between the two passes.
   const uint32_t fillers = 64u / static_cast<uint32_t>(kVol) + 1u < gridDim.x ? 64u / static_cast<uint32_t>(kVol) + 1u : gridDim.x;
   if (incrementalFill && b < fillers) {
-    uint32_t end = 0, myStart = 0;
-    for (int t = 0; t < kVol; ++t) {
-      if (t == tap) myStart = end;
-      end += tapSegment(totals, t);
+    uint32_t mineBefore = 0, mineAll = 0;
+    for (int t = threadIdx.x; t < kVol; t += blockDim.x) {
+      const uint32_t seg = tapSegment(totals, t);
+      mineAll += seg;
+      if (t < tap) mineBefore += seg;
     }
+    const uint32_t end = blockSum(mineAll, scratch);
+    const uint32_t myStart = blockSum(mineBefore, scratch);
     const uint32_t oldEnd = fillState[0];
     const uint32_t gid = (static_cast<uint32_t>(tap) * fillers + b) * kRbThreads + threadIdx.x;
     const uint32_t nThreads = fillers * gridDim.y * kRbThreads;
@@ -589,15 +622,22 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
   // the staging entries first: their latency overlaps that of the sums below
   uint4 s4 = make_uint4(kNone, kNone, kNone, kNone);
   if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<int64_t>(tap) * pitch + first);
+  // write position = segments of the earlier taps + pairs of this tap in earlier chunks: both sums are spread
+  // over the threads and share one reduction (one round of loads instead of a serial walk over the taps)
   uint32_t before = 0;
   for (uint32_t q = threadIdx.x; q < b; q += blockDim.x) before += cnt[static_cast<size_t>(tap) * nBlocks + q];
-  uint32_t pos = blockSum(before, scratch);
-  for (int t = 0; t < tap; ++t) pos += tapSegment(totals, t);
+  for (int t = threadIdx.x; t < tap; t += blockDim.x) before += tapSegment(totals, t);
 
   uint32_t v[kRbItems] = {s4.x, s4.y, s4.z, s4.w};
+  uint32_t mine = 0;
 #pragma unroll
-  for (int j = 0; j < kRbItems; ++j)
+  for (int j = 0; j < kRbItems; ++j) {
     if (first + j >= n) v[j] = kNone;
+    mine += (v[j] != kNone);
+  }
+  uint32_t pos;
+  uint32_t at = blockSumAndScan(before, mine, scratch, &pos);  // one pair of barriers for the sum and the ranks
+  at += pos;
   const bool shuffled = perm && *permShuffled;
   if (shuffled) {  // block-map SubM: the probe stored ranks; rows are perm[rank]
 #pragma unroll
@@ -605,9 +645,6 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
       if (v[j] != kNone) v[j] = perm[v[j]];
   }
   if (!inPlace || shuffled || first + kRbItems > n) mirrorStore(v);
-  uint32_t mine = 0;
-#pragma unroll
-  for (int j = 0; j < kRbItems; ++j) mine += (v[j] != kNone);
   if (masks && mirror && kVol <= 64) {
     // tile masks of the convolution (bit t of masks[r / 64]: some output row of 64-row tile r / 64 has tap t).
     // Mirrored table: this thread's 4 consecutive INPUT rows are output rows under tap kVol-1-tap; a 16-lane row
@@ -617,8 +654,6 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
     if ((lane & 15) == 0 && ((any >> lane) & 0xFFFFull) && first < nbrRows)
       atomicOr(&masks[first >> 6], 1ull << (kVol - 1 - tap));
   }
-  uint32_t total;
-  uint32_t at = pos + blockExclusiveScan(mine, scratch, &total);
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
     if (v[j] != kNone) {
