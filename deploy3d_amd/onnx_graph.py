@@ -13,8 +13,9 @@ the sparse section of such a graph:
 * ``GraphExecutor`` creates one operator per ``TRT_PluginV2`` node through the C ABI, allocates every tensor once
   at its static capacity, links each SPConvMM to the SPConvIdx node that produces its index tensor (several
   convolutions may share one), and enqueues the nodes in topological order on the current stream - no host
-  synchronisation, so a run can be captured in a HIP graph.  Besides plugin nodes it runs ``Add`` (residual sums of
-  two feature tensors); dense 2-D heads are outside its scope and any other op type is refused.
+  synchronisation, so a run can be captured in a HIP graph.  Besides plugin nodes it runs ``Cast`` (voxel means to
+  the backbone's type) and ``Add`` (residual sums of two feature tensors); dense 2-D heads are outside its scope
+  and any other op type is refused.
 """
 import struct
 
@@ -249,18 +250,35 @@ def plugin_node(name, blob, inputs, outputs, version="2.0", node_name=""):
 
 
 def backbone_model(layers, weights, capacities, n_in, in_channels, grid, dtype=torch.float16, batch=1,
-                   densify=False):
+                   densify=False, points=0):
     """The graph the reference's exporter produces for a chain / small DAG of sparse convolutions described by a
     layer table (deploy3d_amd.synth): one SPConvIdx node per indice key, one SPConvMM node per layer, ``Add`` for a
-    two-source layer, optionally a BEVDensify node at the end.  Inputs: feats, coors, num_act, spatial_shape."""
+    two-source layer, optionally a BEVDensify node at the end.  Inputs: feats, coors, num_act, spatial_shape - or,
+    with ``points`` > 0 (the capacity of the point tensor), points [points, in_channels] float, batch_indices,
+    voxel_config and spatial_shape: a SimpleMeanEncoder node then makes the voxels (n_in = its maxNumActOut) and a
+    ``Cast`` brings its float means to the backbone's type (the reference's points -> voxels -> backbone graphs)."""
     from .spconv_index import index_blob
     from .spconv_mm import mm_blob
     elem = _TORCH_TO_ELEM[dtype]
     nd = len(grid)
-    inputs = [Value("feats", elem, [n_in, in_channels]), Value("coors", INT32, [n_in, nd + 1]),
-              Value("num_act", INT32, [1]), Value("spatial_shape", INT32, [batch, 0] + list(grid))]
     nodes = []
-    state = {"input": dict(feats="feats", coors="coors", num="num_act", shape="spatial_shape", cap=n_in,
+    if points:
+        from .simple_mean import simple_mean_blob
+        inputs = [Value("points", FLOAT, [points, in_channels]), Value("batch_indices", INT32, [points]),
+                  Value("voxel_config", FLOAT, [6]), Value("spatial_shape", INT32, [batch, 0] + list(grid))]
+        nodes.append(plugin_node("SimpleMeanEncoder", simple_mean_blob(n_in),
+                                 ["points", "batch_indices", "voxel_config", "spatial_shape"],
+                                 ["voxel_means", "coors", "num_act"], node_name="voxels"))
+        if dtype == torch.float32:
+            first = "voxel_means"
+        else:
+            nodes.append(Node("Cast", ["voxel_means"], ["feats"], dict(to=elem), name="voxel_cast"))
+            first = "feats"
+    else:
+        inputs = [Value("feats", elem, [n_in, in_channels]), Value("coors", INT32, [n_in, nd + 1]),
+                  Value("num_act", INT32, [1]), Value("spatial_shape", INT32, [batch, 0] + list(grid))]
+        first = "feats"
+    state = {"input": dict(feats=first, coors="coors", num="num_act", shape="spatial_shape", cap=n_in,
                            grid=list(grid))}
     keys = {}
     cur = state["input"]
@@ -334,6 +352,9 @@ class GraphExecutor:
                     raise ValueError("%r: TRT_PluginV2 node without name / data attributes" % n)
                 version = n.attrs.get("version", b"2.0")
                 self.plugins[i] = Plugin(bytes(name).decode(), blob, bytes(version).decode())
+            elif n.op_type == "Cast":
+                if n.attrs.get("to") not in _ELEM_TO_TORCH:
+                    raise NotImplementedError("Cast to ONNX element type %r (node %s)" % (n.attrs.get("to"), n.name))
             elif n.op_type != "Add":
                 raise NotImplementedError("op type %s (node %s) is outside the sparse section this executor runs"
                                           % (n.op_type, n.name or n.outputs))
@@ -405,6 +426,11 @@ class GraphExecutor:
                 values[n.outputs[0]] = out
                 plan.append(("add", ins, out))
                 continue
+            if n.op_type == "Cast":
+                out = torch.empty(ins[0].shape, dtype=_ELEM_TO_TORCH[n.attrs["to"]], device=self.device)
+                values[n.outputs[0]] = out
+                plan.append(("cast", ins, out))
+                continue
             p = self.plugins[i]
             in_descs = [TensorDesc.of_tensor(t) for t in ins]
             out_descs = p.output_descs(in_descs)
@@ -430,6 +456,8 @@ class GraphExecutor:
         for step in self._bound["plan"]:
             if step[0] == "add":
                 torch.add(step[1][0], step[1][1], out=step[2])
+            elif step[0] == "cast":
+                step[2].copy_(step[1][0])
             else:
                 _, p, in_descs, out_descs, ins, outs, ws = step
                 p.enqueue(in_descs, out_descs, ins, outs, ws)

@@ -94,3 +94,72 @@ def test_whole_configurations_and_graph_capture(engine, config, n):
             torch.cuda.synchronize()
             _same(y, out, ex.model)
             assert torch.equal(out["bev"], bev)
+
+
+def test_points_to_dense_map_as_one_graph(engine):
+    """All four operators in one graph: SimpleMeanEncoder -> Cast -> SPConvIdx / SPConvMM chain -> BEVDensify.  The
+    graph's outputs equal, bit for bit, the same stages called one by one (which test_gpu_pipeline.py holds against
+    the oracle) - eagerly, with fewer points in the same buffers, and from a HIP-graph replay; the native schedule
+    refuses the Cast."""
+    from deploy3d_amd import layers, onnx_graph, simple_mean_encoder, synth
+    rng = np.random.default_rng(5)
+    n_pts, max_vox = 40000, 20000
+    grid = (16, 96, 96)
+    vcfg = np.array([-9.6, -9.6, -1.0, 0.2, 0.2, 0.25], np.float32)
+    pts = np.empty((n_pts, 5), np.float32)
+    pts[:, 0:2] = rng.normal(0, 4.0, (n_pts, 2))
+    pts[:, 2] = np.where(rng.random(n_pts) < 0.7, rng.uniform(-1.0, -0.4, n_pts), rng.normal(0.5, 0.8, n_pts))
+    pts[:, 3:] = rng.random((n_pts, 2))
+    batch = np.zeros(n_pts, np.int32)
+    batch[rng.integers(0, n_pts, 300)] = -1
+    specs = synth.voxelnet_layers()[:4]
+    weights = [synth.layer_weights(0, i, s) for i, s in enumerate(specs)]
+    caps = layers.plan_capacities(specs, max_vox)
+    model = onnx_graph.backbone_model(specs, weights, caps, max_vox, 5, grid, densify=True, points=n_pts)
+    assert [n.attrs.get("name", n.op_type.encode()) for n in model.nodes[:2]] == [b"SimpleMeanEncoder", b"Cast"]
+    ex = onnx_graph.GraphExecutor(onnx_graph.write_model(model))
+    net = layers.SparseBackbone(specs, weights, caps, overlap=False)
+    d_pts, d_batch = torch.from_numpy(pts).cuda(), torch.from_numpy(batch).cuda()
+    d_cfg = torch.from_numpy(vcfg).cuda()
+    shape = torch.empty((1, 0) + grid, dtype=torch.int32, device="cuda")
+    inputs = dict(points=d_pts, batch_indices=d_batch, voxel_config=d_cfg, spatial_shape=shape)
+
+    def stage_by_stage(vals):
+        """The voxeliser called on its own (coordinates and order exact; its means are sums of fp32 atomics, equal
+        up to the order of addition), then the layer runner and the densifier on the graph's own voxels."""
+        f, c, k = simple_mean_encoder(d_pts, d_batch, d_cfg, shape, max_vox)
+        nv = int(k.item())
+        assert nv == int(vals["num_act"].item()) and torch.equal(c[:nv], vals["coors"][:nv])
+        torch.testing.assert_close(f[:nv], vals["voxel_means"][:nv], rtol=1e-5, atol=1e-6)
+        y = net.forward(layers.SparseTensor(vals["voxel_means"].half(), vals["coors"], vals["num_act"], list(grid), 1))
+        return y, layers.densify(y).clone()
+
+    for drop in (0, n_pts // 2):
+        d_batch.copy_(torch.from_numpy(batch))
+        if drop:
+            d_batch[:drop] = -1                          # fewer points, same buffers
+        out = ex.run(**inputs)
+        torch.cuda.synchronize()
+        y, bev = stage_by_stage(ex._bound["values"])
+        torch.cuda.synchronize()
+        assert 1000 < int(y.num_act.item()) < max_vox
+        _same(y, out, ex.model)
+        assert torch.equal(out["bev"], bev)
+    with pytest.raises(NotImplementedError):
+        ex.run_scheduled(**inputs)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        out = ex.run(**inputs)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            out = ex.run(**inputs)
+        for _ in range(2):
+            out["bev"].zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            y, bev = stage_by_stage(ex._bound["values"])
+            torch.cuda.synchronize()
+            _same(y, out, ex.model)
+            assert torch.equal(out["bev"], bev)
