@@ -1212,7 +1212,11 @@ bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_
 #pragma unroll
   for (int e = 0; e < kNearGroup; ++e) {
     const unsigned long long want = masks[e][threadIdx.x];
-    orRuns(records, ((present >> e) & 1u) && want ? rec[e] : kNone, want);
+    const bool any = ((present >> e) & 1u) && want;
+    // wavefront-uniform: most of the twelve group members get no candidate from any of a wavefront's 64 inputs
+    // (a strided kernel reaches two of the three levels, and neighbouring inputs share their bricks)
+    if (__ballot(any) == 0ull) continue;
+    orRuns(records, any ? rec[e] : kNone, want);
   }
 }
 
