@@ -28,6 +28,12 @@ typedef int32_t (*count_fn)(void);
 typedef const char* (*name_fn)(int32_t);
 typedef int32_t (*link_fn)(d3d_plugin*, d3d_plugin*);
 typedef int32_t (*option_fn)(d3d_plugin*, int32_t, int64_t);
+typedef int32_t (*sched_create_fn)(int32_t, d3d_schedule**);
+typedef int32_t (*sched_add_fn)(d3d_schedule*, d3d_plugin*, const d3d_tensor_desc*, int32_t, const d3d_tensor_desc*,
+                                int32_t, const void* const*, void* const*, void*, size_t, int32_t, const int32_t*,
+                                int32_t);
+typedef int32_t (*sched_size_fn)(const d3d_schedule*);
+typedef void (*sched_destroy_fn)(d3d_schedule*);
 
 int main(int argc, char** argv) {
   CHECK(argc == 2);
@@ -49,8 +55,13 @@ int main(int argc, char** argv) {
   name_fn op_name = (name_fn)dlsym(lib, "d3d_op_name");
   link_fn link_rulebook = (link_fn)dlsym(lib, "d3d_link_rulebook");
   option_fn set_option = (option_fn)dlsym(lib, "d3d_set_option");
+  sched_create_fn sched_create = (sched_create_fn)dlsym(lib, "d3d_schedule_create");
+  sched_add_fn sched_add = (sched_add_fn)dlsym(lib, "d3d_schedule_add");
+  sched_size_fn sched_size = (sched_size_fn)dlsym(lib, "d3d_schedule_size");
+  sched_destroy_fn sched_destroy = (sched_destroy_fn)dlsym(lib, "d3d_schedule_destroy");
   CHECK(create && clone && destroy && ser_size && serialize && num_outputs && output_dims && last_error &&
-        plugin_type && num_ops && op_name && link_rulebook && set_option);
+        plugin_type && num_ops && op_name && link_rulebook && set_option && sched_create && sched_add &&
+        sched_size && sched_destroy);
 
   CHECK(num_ops() >= 5);
   CHECK(strcmp(op_name(2), "SPConvIdx3d") == 0);
@@ -100,6 +111,25 @@ int main(int argc, char** argv) {
   CHECK(set_option(mm, D3D_OPT_PERSISTENT_INDEX, 1) == D3D_ERR_UNSUPPORTED && strlen(last_error()) > 0);
   CHECK(set_option(p, 12345, 1) == D3D_ERR_UNSUPPORTED);
   CHECK(set_option(NULL, D3D_OPT_PERSISTENT_INDEX, 1) == D3D_ERR_BAD_ARG);
+  /* a one-lane schedule is pure bookkeeping (no stream, no event): steps are copied, bad steps refused */
+  d3d_schedule* sched = NULL;
+  CHECK(sched_create(0, &sched) == D3D_ERR_BAD_ARG && sched == NULL);
+  CHECK(sched_create(1, &sched) == D3D_OK && sched && sched_size(sched) == 0);
+  {
+    d3d_tensor_desc outs[5];
+    const void* in_ptrs[3] = {NULL, NULL, NULL};
+    void* out_ptrs[5] = {NULL, NULL, NULL, NULL, NULL};
+    const int32_t first = 0, self = 2;   /* the third step would be step 2 */
+    for (int i = 0; i < 5; ++i) CHECK(output_dims(p, i, in, 3, &outs[i]) == D3D_OK);
+    CHECK(sched_add(sched, p, in, 3, outs, 5, in_ptrs, out_ptrs, NULL, 0, 0, NULL, 0) == 0);
+    CHECK(sched_add(sched, q, in, 3, outs, 5, in_ptrs, out_ptrs, NULL, 0, 0, &first, 1) == 1);
+    CHECK(sched_add(sched, p, in, 3, outs, 4, in_ptrs, out_ptrs, NULL, 0, 0, NULL, 0) == D3D_ERR_BAD_ARG);
+    CHECK(sched_add(sched, p, in, 3, outs, 5, in_ptrs, out_ptrs, NULL, 0, 1, NULL, 0) == D3D_ERR_BAD_ARG);
+    CHECK(sched_add(sched, p, in, 3, outs, 5, in_ptrs, out_ptrs, NULL, 0, 0, &self, 1) == D3D_ERR_BAD_ARG);
+    CHECK(sched_size(sched) == 2);
+  }
+  sched_destroy(sched);
+  sched_destroy(NULL);
   destroy(mm);
   destroy(q);
   destroy(p);
