@@ -130,7 +130,8 @@ class SparseBackbone:
     kernels of later stages run beside the MFMA kernels of earlier ones.  A SubM rulebook is ordered behind the
     strided rulebook that wrote its coordinates through an event of the MAIN stream, recorded where the main
     stream waited for that rulebook (an event edge straight from one side stream to the other made
-    hipStreamEndCapture crash in the runtime).  The side streams fork from and join into the caller's current
+    hipStreamEndCapture crash in the runtime).  A strided rulebook in turn starts behind the SubM rulebook of the
+    stage before it, which the convolutions need first.  The side streams fork from and join into the caller's current
     stream, so a forward pass can still be captured into one HIP graph (it then holds parallel branches).
 
     ``index_tensors=False`` tells the rulebook operators that nothing outside this runner reads their index tensors
@@ -173,6 +174,7 @@ class SparseBackbone:
         inputs = {}
         pending = {}
         strided_coords = {}  # coordinate tensor written by a strided rulebook -> main-stream event after its wait
+        subm_done = None     # main-stream event behind the wait for the latest SubM rulebook on strided coordinates
         outs = {"input": x}
         cur = x
         for spec, lyr in zip(self.specs, self.layers):
@@ -193,16 +195,25 @@ class SparseBackbone:
                     # order behind the strided rulebook that wrote these coordinates, carried by an event of the
                     # main stream (recorded when the main stream waited for that rulebook)
                     st.wait_event(strided_coords[id(inp.coors)])
+                if not subm and subm_done is not None:
+                    # The SubM rulebook of the stage before (same input coordinates) is what the convolutions wait
+                    # for next; this one is not needed before that stage's convolutions are through.  Running both at
+                    # once stretches both, so this one starts when that one is done - again through an event of the
+                    # main stream (0.75 -> 0.72 ms per pass of the VoxelNet backbone; making the FIRST strided
+                    # rulebook wait for the input's SubM rulebook as well measured slower).
+                    st.wait_event(subm_done)
                 with torch.cuda.stream(st):
                     rb = rulebooks[key] = lyr.build_rulebook(inp)
                     pending[key] = torch.cuda.Event()
                     pending[key].record(st)
             if key in pending:
                 main.wait_event(pending.pop(key))
+                seen = torch.cuda.Event()
+                seen.record(main)
                 if not spec["subm"]:
-                    seen = torch.cuda.Event()
-                    seen.record(main)
                     strided_coords[id(rulebooks[key].out_coors)] = seen
+                elif id(inp.coors) in strided_coords:
+                    subm_done = seen
             cur = lyr.forward(inp, rulebooks)
             outs[spec["name"]] = cur
         self.rulebooks = rulebooks
