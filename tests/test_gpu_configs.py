@@ -130,6 +130,41 @@ def test_native_schedule_equals_the_stream_runner(engine, config, n, index_tenso
     assert e.value.status == -1
 
 
+def test_schedule_on_one_lane_and_back_to_back_runs(engine):
+    """A schedule built by hand on a single lane (the caller's stream only, no stream or event of its own), run
+    several times back to back without a synchronisation in between on a non-default stream: every run gives the
+    step-by-step result, and work enqueued behind a run on that stream sees the run's output."""
+    from deploy3d_amd import layers, synth
+    from deploy3d_amd.plugin import Schedule
+    cfg = synth.config2(20000)
+    specs, weights = cfg["layers"], cfg["weights"]
+    n = len(cfg["coords"])
+    caps = layers.plan_capacities(specs, n, layers.measure_output_counts(specs, cfg["coords"], cfg["grid"]))
+    net = layers.SparseBackbone(specs, weights, caps, overlap=False)
+    x = layers.make_input(cfg["coords"], cfg["feats"], cfg["grid"])
+    y = net.forward(x)
+    torch.cuda.synchronize()
+    want = y.feats.clone()
+    lyr, rb = net.layers[0], net.rulebooks[specs[0]["key"]]
+    sched = Schedule(lanes=1)
+    st = lyr._idx_state
+    a = sched.add(lyr.idx_plugin, st["in_descs"], st["out_descs"], [x.coors, x.num_act, None], st["outs"], st["ws"])
+    st = lyr._mm_state
+    b = sched.add(lyr.mm_plugin, st["in_descs"], st["out_descs"],
+                  [x.feats, rb.num_act_in, rb.num_act_out, rb.index, rb.num_index], [st["out"]], after=[a])
+    assert (a, b) == (0, 1)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        copies = []
+        for _ in range(4):
+            y.feats.zero_()
+            sched.run()
+            copies.append(y.feats.clone())      # ordered behind the run on the same stream
+    stream.synchronize()
+    for c in copies:
+        assert torch.equal(c, want)
+
+
 def test_down_up_chain_with_inverse_convolution(engine):
     """An encoder-decoder wiring through the layer runner: strided down (key d), SubM at the lower resolution, then
     the inverse convolution of key d back onto the input sites, then a SubM that shares the first layer's key.  The
