@@ -135,7 +135,8 @@ vxRank(const unsigned long long* __restrict__ table, const uint32_t* __restrict_
   }
   if (threadIdx.x == 0) {
     // the total is published with a returning device-scope atomic (performed where every XCD sees it once the
-    // result is back); only then is the ticket taken
+    // result is back); only then is the ticket taken.  An acquire-release ticket instead (a device-scope release
+    // per workgroup) measured 8.2 -> 13.8 us for this kernel on 100 000 points.
     uint32_t old = __hip_atomic_exchange(&chunkBase[blockIdx.x], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(old)::"memory");
     isLast = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nChunks - 1 ? 1u : 0u;
