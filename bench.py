@@ -51,9 +51,10 @@ def r_to(a, dtype):
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(t).float().numpy()
 
 
-def cpu_pass(cfg, threads):
+def cpu_pass(cfg, threads, rulebooks_out=None):
     """One pass of the workload through the CPU oracle (fp32 accumulation on storage-rounded operands; int32
-    accumulation + the requantize rule for int8).  Returns (rulebook s, conv s, final coords, final features)."""
+    accumulation + the requantize rule for int8).  Returns (rulebook s, conv s, final coords, final features);
+    ``rulebooks_out`` (a dict) receives the oracle's rulebook per indice key, with the coordinates it was built on."""
     import numpy as np
     from oracle import oracle
     dtype = cfg["dtype"]
@@ -88,6 +89,7 @@ def cpu_pass(cfg, threads):
                 rb["out_coors"] = rb["out_coors"][:rb["num_act_out"]].copy()
                 rb["out_grid"] = og
             t_rb += time.perf_counter() - t0
+            rb["in_coors"] = x["coords"]
             rulebooks[spec["key"]] = rb
         t0 = time.perf_counter()
         if int8:
@@ -104,6 +106,8 @@ def cpu_pass(cfg, threads):
         t_conv += time.perf_counter() - t0
         cur = dict(feats=y, coords=rb["out_coors"], grid=rb["out_grid"])
         outs[spec["name"]] = cur
+    if rulebooks_out is not None:
+        rulebooks_out.update(rulebooks)
     return t_rb, t_conv, cur["coords"], cur["feats"]
 
 

@@ -345,6 +345,49 @@ def test_config3_backbone_full_size_properties(engine):
     assert float((lhs - rhs).abs().max()) <= 2e-2 * float(rhs.pow(2).mean().sqrt()) + 4e-3
 
 
+def _bench_module():
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    return bench
+
+
+@pytest.mark.parametrize("config,min_pairs", [(3, 10_000_000), (5, 3_000_000)])
+def test_backbones_at_full_size_against_the_oracle(engine, config, min_pairs):
+    """Configs 3 and 5 at their stated sizes (120 000 voxels - the workload of the bench line - and 250 000) against
+    one full pass of the CPU oracle with fp32 accumulation (the pass bench.py times as its CPU baseline): every
+    rulebook bit for bit in canonical form (10.3 M pairs for config 3, 3.5 M for config 5) and the final features within 2e-2 * rms on
+    identical coordinates."""
+    import os
+    bench = _bench_module()
+    from deploy3d_amd import synth
+    cfg = synth.config3() if config == 3 else synth.config5()
+    net, x, y = run_gpu_chain(cfg)
+    ref_rulebooks = {}
+    _, _, ref_coords, ref_feats = bench.cpu_pass(cfg, min(16, os.cpu_count() or 1), ref_rulebooks)
+    assert set(ref_rulebooks) == set(net.rulebooks)
+    pairs = 0
+    for key, rb in net.rulebooks.items():
+        orb = ref_rulebooks[key]
+        n_out = int(rb.num_act_out.item())
+        assert n_out == orb["num_act_out"], key
+        c_got, t_got = chain.canonical_pairs(rb.index.cpu().numpy(), int(rb.num_index.item()), rb.in_coors.cpu().numpy(),
+                                             int(rb.num_act_in.item()), rb.out_coors.cpu().numpy(), n_out)
+        c_ref, t_ref = chain.canonical_pairs(orb["index"], orb["num_index"], orb["in_coors"], len(orb["in_coors"]),
+                                             orb["out_coors"], orb["num_act_out"])
+        np.testing.assert_array_equal(c_got, c_ref, err_msg=key)
+        np.testing.assert_array_equal(t_got, t_ref, err_msg=key)
+        pairs += len(t_got)
+    assert pairs > min_pairs
+    n = int(y.num_act.item())
+    gc, gf = chain.sort_rows(y.coors[:n].cpu().numpy(), y.feats[:n].float().cpu().numpy())
+    rc, rf = chain.sort_rows(ref_coords, np.asarray(ref_feats, dtype=np.float32))
+    assert np.array_equal(gc, rc)
+    rms = float(np.sqrt(np.mean(rf.astype(np.float64) ** 2)))
+    assert float(np.abs(gf - rf).max()) <= 2e-2 * rms
+
+
 def test_config3_graph_replay_matches_eager(engine):
     """The whole backbone captured in a HIP graph: three replays, each equal to the eager result."""
     from deploy3d_amd import layers, synth
@@ -471,6 +514,15 @@ def test_config4_int8_backbone_full_size(engine):
             want = oracle.requantize(acc.astype(np.int32), m, bq, bool(spec.get("relu")))
             np.testing.assert_array_equal(q[rows].cpu().numpy(), want, err_msg=spec["name"])
         prev = spec["name"]
+    # and the whole pass against the oracle's int8 pass (int32 accumulation, the same requantize rule): the final
+    # tensor of all 13 layers, every row, bit for bit
+    import os
+    _, _, ref_coords, ref_feats = _bench_module().cpu_pass(cfg, min(16, os.cpu_count() or 1))
+    n_out = int(y.num_act.item())
+    gc, gf = chain.sort_rows(y.coors[:n_out].cpu().numpy(), first[cfg["layers"][-1]["name"]][:n_out].cpu().numpy())
+    rc, rf = chain.sort_rows(ref_coords, np.asarray(ref_feats))
+    assert np.array_equal(gc, rc)
+    np.testing.assert_array_equal(gf, rf)
 
 
 def test_config5_full_size_first_layers_vs_oracle(engine):
