@@ -20,6 +20,8 @@
 // Gathers and index loads are buffer loads: an absent neighbour (-1) or a row past the input produces an
 // out-of-range offset, for which the hardware delivers zeros - no zero row, no select, one VALU per gather.
 #pragma once
+#include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 #include "conv_kernels.h"
@@ -64,7 +66,7 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
   constexpr int PER = TM / 64;                                 // tile masks per workgroup tile
   constexpr int ROWSHIFT = CIN * ES == 64 ? 6 : (CIN * ES == 128 ? 7 : 8);
   static_assert(ES == 2 && (CS == 32 || CS == 64) && CIN % CS == 0 && WM % RPI == 0 && TM % 64 == 0, "shape");
-  static_assert((1 << ROWSHIFT) == CIN * ES && WCH % 64 == 0 && MT % 2 == 0 && MT * NT * 4 <= 128, "shape");
+  static_assert((1 << ROWSHIFT) == CIN * ES && WCH % 64 == 0 && MT >= 2 && MT * NT * 4 <= 128, "shape");
   using F = u32x4;
   using Acc = typename Mfma<T>::Acc;
 
@@ -298,6 +300,9 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
   int wbuf = 0;
   auto step = [&](int a, auto slotTag, F (&curW)[KK][NT], F (&nxtW)[KK][NT]) __attribute__((always_inline)) -> bool {
     constexpr int SLOT = decltype(slotTag)::value;
+    // The two register sets alternate from group to group, across steps as well: with an odd number of groups
+    // per step the set a group uses flips with the parity of the step (SLOT is that parity).
+    constexpr int PAR = (MT & 1) ? SLOT : 0;
     constexpr int WREADS = (NQ + MT - 1) / MT;      // weight fragment reads per group
     // Loads ride behind MFMAs: the GPM gathers of a group behind its first GPM MFMAs, and the remaining
     // ("free") MFMA slots of the step, in order, carry the index load and then the WL weight loads.
@@ -315,18 +320,18 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
     const int nextBuf = wbuf + 1 == NWB ? 0 : wbuf + 1;
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-      F(&cur)[KK] = rowBuf[m & 1];
-      F(&nxt)[KK] = rowBuf[(m + 1) & 1];
-      int32_t(&ix)[GPM] = ixBuf[m & 1];
+      F(&cur)[KK] = rowBuf[(m + PAR) & 1];
+      F(&nxt)[KK] = rowBuf[(m + 1 + PAR) & 1];
+      int32_t(&ix)[GPM] = ixBuf[(m + PAR) & 1];
       if (m + 1 < MT) {
         if constexpr (!(DBG & 4)) readRowGroup(nxt, m + 1, SLOT);
-        readIndex(a + 2, m + 1, ixBuf[(m + 1) & 1]);
+        readIndex(a + 2, m + 1, ixBuf[(m + 1 + PAR) & 1]);
       } else {
         // everything issued before this step has landed: the rows of the next step, this wavefront's part of
         // the weight slice of the step after next, the indices of the step after that
         waitVmcnt<((DBG & 1) ? 0 : (MT - 1) * GPM) + extraBeforeWait>();
         if constexpr (!(DBG & 4)) readRowGroup(nxt, 0, SLOT ^ 1);
-        readIndex(a + 3, 0, ixBuf[0]);
+        readIndex(a + 3, 0, ixBuf[(m + 1 + PAR) & 1]);
       }
 #pragma unroll
       for (int e = m * WREADS; e < (m + 1) * WREADS && e < NQ; ++e)
@@ -411,26 +416,43 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
 // tile halves.  32 -> 32 takes 8 wavefronts as well (two workgroups of 78 KB per CU, 16 wavefronts): 38 us against
 // 41 with 4, 40 with three 4-wavefront workgroups per CU, 41 with 128-row wavefront tiles; with gathers and MFMAs
 // both taken out of it the kernel still runs 27 us on that layer (25 with the table reads served from cache), so
-// what is left is the per-step bookkeeping of a 32-channel step, not a memory or matrix limit.  Layers with few rows (the 128-channel stages: 47 000 rows are
-// 186 tiles of 256 rows for 256 CUs) pick the workgroup size whose tile count loads the CUs most evenly: the
-// time of a layer that fits one round is that of ONE tile, so 248 tiles of 192 rows beat 186 of 256.
+// what is left is the per-step bookkeeping of a 32-channel step, not a memory or matrix limit.  Layers with few
+// rows (the 128-channel stages: 47 000 rows are 186 tiles of 256 rows for 256 CUs) pick the workgroup shape by a
+// cost model of one tile's step on its CU: the time of a layer that fits one round is that of ONE tile, so 248
+// tiles of 192 rows beat 186 of 256 (48 us against 55), and four wavefronts of 48 rows - one per SIMD, three
+// 16-row groups each - beat six of 32 rows, which load two SIMDs twice as much as the others (45 us against 48).
 template <class T, int CIN, int COUT>
 int32_t launchPipeShape(const ConvArgs& a, hipStream_t stream) {
   if constexpr (CIN == 64 && COUT == 64) {
     return launchPipeCfg<T, CIN, COUT, 4, 8>(a, stream);
   } else if constexpr (COUT >= 128) {
-    int best = 8;
+    // candidates (rows per wavefront, wavefronts): cost = rounds of tiles over the 256 CUs x cycles of one step of
+    // a tile on its CU, the larger of the MFMA issue of the busiest SIMD (wavefronts are dealt to the four SIMDs
+    // in turn; 16 cycles per MFMA, COUT / 16 * CS / 32 MFMAs per 16 rows) and the LDS traffic at 128 bytes per
+    // cycle (every wavefront reads the step's whole weight slice; every row is written once and read once)
+    static const int kCand[4][2] = {{32, 8}, {32, 6}, {32, 4}, {48, 4}};
+    constexpr int CSTEP = CIN > 64 ? 64 : CIN;
+    int best = 0;
     int64_t bestCost = 0;
-    for (int waves = 8; waves >= 4; waves -= 2) {
-      const int64_t tm = 32 * waves, tiles = (a.outRows + tm - 1) / tm;
-      const int64_t cost = (tiles + 255) / 256 * tm;  // rows the busiest CU multiplies
-      if (waves == 8 || cost < bestCost) {
-        best = waves;
+    for (int c = 0; c < 4; ++c) {
+      const int64_t rows = kCand[c][0], waves = kCand[c][1], tm = rows * waves, tiles = (a.outRows + tm - 1) / tm;
+      const int64_t mfma = (waves + 3) / 4 * rows / 16 * (COUT / 16) * (CSTEP / 32) * 16;
+      const int64_t lds = (waves * CSTEP * COUT * 2 + tm * CSTEP * 2 * 2) / 128;
+      const int64_t cost = (tiles + 255) / 256 * (mfma > lds ? mfma : lds);
+      if (c == 0 || cost < bestCost) {
+        best = c;
         bestCost = cost;
       }
     }
-    if (best == 6) return launchPipeCfg<T, CIN, COUT, 2, 6>(a, stream);
-    if (best == 4) return launchPipeCfg<T, CIN, COUT, 2, 4>(a, stream);
+    if (const char* force = debugEnv("D3D_CONV_PIPE_SHAPE")) {  // "rows,wavefronts" of one candidate (tests)
+      for (int c = 0; c < 4; ++c)
+        if (std::atoi(force) == kCand[c][0] && std::strchr(force, ',') &&
+            std::atoi(std::strchr(force, ',') + 1) == kCand[c][1])
+          best = c;
+    }
+    if (best == 1) return launchPipeCfg<T, CIN, COUT, 2, 6>(a, stream);
+    if (best == 2) return launchPipeCfg<T, CIN, COUT, 2, 4>(a, stream);
+    if (best == 3) return launchPipeCfg<T, CIN, COUT, 3, 4>(a, stream);
     return launchPipeCfg<T, CIN, COUT, 2, 8>(a, stream);
   } else if constexpr (CIN == 32 && COUT == 32) {
     return launchPipeCfg<T, CIN, COUT, 4, 8>(a, stream);

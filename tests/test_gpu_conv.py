@@ -269,6 +269,21 @@ def test_mfma_tile_sizes(engine, monkeypatch, tile_rows, cin, cout):
     run_case(3001, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, "float16", True, relu=True)
 
 
+@pytest.mark.parametrize("shape", ["32,8", "32,6", "32,4", "48,4"])
+@pytest.mark.parametrize("cin,cout,dtype", [(32, 128, "float16"), (64, 128, "float16"), (128, 128, "float16"),
+                                            (128, 128, "bfloat16")])
+def test_pipelined_tile_shapes_of_wide_layers(engine, monkeypatch, shape, cin, cout, dtype):
+    """The four workgroup shapes (rows per wavefront, wavefronts) the pipelined kernel chooses from for 128 output
+    channels by row count - 48-row wavefronts (three 16-row groups: the register sets alternate across steps) among
+    them - each forced on a SubM layer (tile masks) and a strided one, and once on a layer with more tiles than
+    workgroups, where the pipeline runs across tiles."""
+    monkeypatch.setenv("D3D_CONV_PIPE_SHAPE", shape)
+    run_case(9001, (12, 48, 40), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, dtype, True, relu=True, cap_extra=50)
+    if cin == 64:
+        run_case(5000, (12, 48, 40), (3, 3, 3), (2, 2, 2), (1, 1, 1), cin, cout, dtype, False)
+        run_case(70000, (16, 200, 200), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, dtype, True, relu=True)
+
+
 @pytest.mark.parametrize("cfg", ["off", "4,8,2", "2,8,3", "2,8,2", "4,4,2", "4,4,3", "4,8,3,1", "2,8,3,1"])
 @pytest.mark.parametrize("cin,cout", [(16, 32), (32, 32), (32, 64), (64, 64), (64, 128), (128, 128), (128, 16)])
 def test_staged_configurations(engine, monkeypatch, cfg, cin, cout):
