@@ -67,6 +67,7 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
   constexpr int ROWSHIFT = CIN * ES == 64 ? 6 : (CIN * ES == 128 ? 7 : 8);
   static_assert(ES == 2 && (CS == 32 || CS == 64) && CIN % CS == 0 && WM % RPI == 0 && TM % 64 == 0, "shape");
   static_assert((1 << ROWSHIFT) == CIN * ES && WCH % 64 == 0 && MT >= 2 && MT * NT * 4 <= 128, "shape");
+  static_assert(WM < 64 || WM % 64 == 0, "an index load covers 64 rows: a wavefront tile is below 64 rows or whole multiples");
   using F = u32x4;
   using Acc = typename Mfma<T>::Acc;
 
