@@ -415,7 +415,7 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
 // which read half the weight fragments per MFMA, measured slower on a 64 -> 64 layer: 68 us against 58 - one
 // wavefront per SIMD has nobody to hide its waits); 128 output channels double the accumulators, so the wavefront
 // tile halves.  32 -> 32 takes 8 wavefronts as well (two workgroups of 78 KB per CU, 16 wavefronts): 38 us against
-// 41 with 4, 40 with three 4-wavefront workgroups per CU, 41 with 128-row wavefront tiles; with gathers and MFMAs
+// 41 with 4, 40 with three 4-wavefront workgroups per CU, 41 with 128-row and 42 with 48-row wavefront tiles; with gathers and MFMAs
 // both taken out of it the kernel still runs 27 us on that layer (25 with the table reads served from cache), so
 // what is left is the per-step bookkeeping of a 32-channel step, not a memory or matrix limit.  Layers with few
 // rows (the 128-channel stages: 47 000 rows are 186 tiles of 256 rows for 256 CUs) pick the workgroup shape by a
