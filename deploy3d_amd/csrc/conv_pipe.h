@@ -418,33 +418,32 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
 // 41 with 4, 40 with three 4-wavefront workgroups per CU, 41 with 128-row and 42 with 48-row wavefront tiles; with gathers and MFMAs
 // both taken out of it the kernel still runs 27 us on that layer (25 with the table reads served from cache), so
 // what is left is the per-step bookkeeping of a 32-channel step, not a memory or matrix limit.  Layers with few
-// rows (the 128-channel stages: 47 000 rows are 186 tiles of 256 rows for 256 CUs) pick the workgroup shape by a
-// cost model of one tile's step on its CU: the time of a layer that fits one round is that of ONE tile, so 248
-// tiles of 192 rows beat 186 of 256 (48 us against 55), and four wavefronts of 48 rows - one per SIMD, three
-// 16-row groups each - beat six of 32 rows, which load two SIMDs twice as much as the others (45 us against 48).
+// rows (the 128-channel stages: 47 000 rows are 186 tiles of 256 rows for 256 CUs) pick the workgroup shape by
+// tile count: the time of a layer that fits one round is that of ONE tile, so 248 tiles of 192 rows beat 186 of
+// 256 (48 us against 55), and there four wavefronts of 48 rows - one per SIMD, three 16-row groups each - beat
+// six of 32 rows (45 us against 48).
 template <class T, int CIN, int COUT>
 int32_t launchPipeShape(const ConvArgs& a, hipStream_t stream) {
   if constexpr (CIN == 64 && COUT == 64) {
     return launchPipeCfg<T, CIN, COUT, 4, 8>(a, stream);
   } else if constexpr (COUT >= 128) {
-    // candidates (rows per wavefront, wavefronts): cost = rounds of tiles over the 256 CUs x cycles of one step of
-    // a tile on its CU, the larger of the MFMA issue of the busiest SIMD (wavefronts are dealt to the four SIMDs
-    // in turn; 16 cycles per MFMA, COUT / 16 * CS / 32 MFMAs per 16 rows) and the LDS traffic at 128 bytes per
-    // cycle (every wavefront reads the step's whole weight slice; every row is written once and read once)
+    // 8, 6 or 4 wavefronts of 32 rows: the workgroup size whose tiles load the busiest CU least (rounds of tiles
+    // over the 256 CUs x rows per tile).  A layer that fits ONE round of 192-row tiles takes them as four
+    // wavefronts of 48 rows - one per SIMD - instead of six of 32, which load two SIMDs twice as much as the
+    // others (conv4_x: 45 us against 48); over several rounds the eight-wavefront shapes hide their waits better
+    // (a 64 -> 128 layer of 10 rounds: 105 us with 8 x 32 rows, 138 us with 4 x 48).
     static const int kCand[4][2] = {{32, 8}, {32, 6}, {32, 4}, {48, 4}};
-    constexpr int CSTEP = CIN > 64 ? 64 : CIN;
     int best = 0;
     int64_t bestCost = 0;
-    for (int c = 0; c < 4; ++c) {
-      const int64_t rows = kCand[c][0], waves = kCand[c][1], tm = rows * waves, tiles = (a.outRows + tm - 1) / tm;
-      const int64_t mfma = (waves + 3) / 4 * rows / 16 * (COUT / 16) * (CSTEP / 32) * 16;
-      const int64_t lds = (waves * CSTEP * COUT * 2 + tm * CSTEP * 2 * 2) / 128;
-      const int64_t cost = (tiles + 255) / 256 * (mfma > lds ? mfma : lds);
+    for (int c = 0; c < 3; ++c) {
+      const int64_t tm = kCand[c][0] * kCand[c][1], tiles = (a.outRows + tm - 1) / tm;
+      const int64_t cost = (tiles + 255) / 256 * tm;  // rows the busiest CU multiplies
       if (c == 0 || cost < bestCost) {
         best = c;
         bestCost = cost;
       }
     }
+    if (best == 1 && (a.outRows + 191) / 192 <= 256) best = 3;
     if (const char* force = debugEnv("D3D_CONV_PIPE_SHAPE")) {  // "rows,wavefronts" of one candidate (tests)
       for (int c = 0; c < 4; ++c)
         if (std::atoi(force) == kCand[c][0] && std::strchr(force, ',') &&
