@@ -65,12 +65,13 @@ struct RbWorkspace {
   uint32_t nChunks;
   uint32_t slots;         // hash slots (power of two)
   uint32_t nBlocks;       // input chunks per tap
+  uint32_t cntPitch;      // 16-bit entries per tap row of cnt (a multiple of 8)
   int64_t pitch;          // row pitch of staging, a multiple of the chunk size
   size_t table;           // hash: u64 [slots] key<<32 | value;  block map: records [nRecords]
   size_t ids;             // hash: u32 [slots] output row of an occupied slot (strided only);  block map: perm [cap] (SubM)
   size_t staging;         // u32 [kVol, pitch] per (tap, input): slot, then output row, or ~0
   size_t ownCnt;          // hash: u32 [kVol, nBlocks] owned outputs per (tap, chunk) (strided only);  block map: chunk totals
-  size_t cnt;             // u32 [kVol, nBlocks] valid pairs per (tap, chunk)
+  size_t cnt;             // u16 [kVol, cntPitch] valid pairs per (tap, block of 256 or 1024 inputs)
   size_t totals;          // u32 [2, kVol]  valid pairs per tap; owned outputs per tap
   size_t total;           // bytes
 };

@@ -291,6 +291,9 @@ __device__ __forceinline__ bool tapTarget(const RbGeom& g, const int c[5], const
 // one word of its tap spends longer queueing there than working (1 400 workgroups: 25 us).
 constexpr int kTotalSlots = 8;
 
+// Pairs per (tap, block of 256 or 1024 inputs): at most 1024, kept in 16 bits so that a row of counts is short.
+typedef uint16_t RbCount;
+
 __device__ __forceinline__ uint32_t tapPairs(const uint32_t* __restrict__ totals, int tap) {
   const uint4 a = *reinterpret_cast<const uint4*>(totals + tap * kTotalSlots);
   const uint4 b = *reinterpret_cast<const uint4*>(totals + tap * kTotalSlots + 4);
@@ -300,14 +303,15 @@ __device__ __forceinline__ uint32_t tapSegment(const uint32_t* __restrict__ tota
   return (tapPairs(totals, tap) + (kSegment - 1)) & ~static_cast<uint32_t>(kSegment - 1);
 }
 
-// Publishes the number of flagged items of this workgroup for its tap; `slots` = kTotalSlots for the pair totals,
-// 1 for a plain array of per-tap sums.
-__device__ __forceinline__ void publishCount(uint32_t mine, uint32_t* scratch, uint32_t* cnt, uint32_t nBlocks,
+// Publishes the number of flagged items of this workgroup for its tap in cnt (row pitch nBlocks) and, when `totals` is
+// given, adds it to the per-tap sums there (`slots` partial sums per tap).
+template <class Count>
+__device__ __forceinline__ void publishCount(uint32_t mine, uint32_t* scratch, Count* cnt, uint32_t nBlocks,
                                              uint32_t* totals, int slots) {
   const uint32_t total = blockSum(mine, scratch);
   if (threadIdx.x == 0) {
-    cnt[static_cast<size_t>(blockIdx.y) * nBlocks + blockIdx.x] = total;
-    if (total) atomicAdd(&totals[blockIdx.y * slots + blockIdx.x % slots], total);
+    cnt[static_cast<size_t>(blockIdx.y) * nBlocks + blockIdx.x] = static_cast<Count>(total);
+    if (total && totals) atomicAdd(&totals[blockIdx.y * slots + blockIdx.x % slots], total);
   }
 }
 
@@ -328,7 +332,7 @@ rbSubmInsert(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restr
 __global__ void __launch_bounds__(kRbThreads)
 rbSubmProbe(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
             int64_t pitch, const unsigned long long* __restrict__ table, uint32_t mask, uint32_t* __restrict__ staging,
-            uint32_t* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
+            RbCount* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
   const int tap = blockIdx.y;
@@ -485,7 +489,7 @@ rbConvAssign(RbGeom g, const int32_t* __restrict__ numActIn, int64_t cap, int64_
 // (reference: hashOutIndexKernel, index.cu:158-172), plus per-(tap, chunk) counts.
 __global__ void __launch_bounds__(kRbThreads)
 rbConvResolve(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, const uint32_t* __restrict__ ids,
-              uint32_t* __restrict__ staging, int32_t maxNumActOut, uint32_t* __restrict__ cnt, uint32_t nBlocks,
+              uint32_t* __restrict__ staging, int32_t maxNumActOut, RbCount* __restrict__ cnt, uint32_t nBlocks,
               uint32_t* totals) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
@@ -513,62 +517,290 @@ rbConvResolve(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, 
 
 // ---------------------------------------------------------------------------
 // Compaction (reference: Valid_Counter scan + outputIndexPadOrganizeKernel +
-// indexOrganizeKernel, index.cu:123-156, :352-366).  Workgroup (chunk, tap)
+// indexOrganizeKernel, index.cu:123-156, :352-366).  Workgroup (span, tap)
 // writes the valid pairs of its inputs at
-//   segment start of the tap  +  pairs of that tap in earlier chunks  +  rank.
+//   segment start of the tap  +  pairs of that tap in earlier spans  +  rank.
+// Both sums come from the per-(tap, block) counts the probe pass left in `cnt` with plain stores
+// (cnt[tap * cntPitch + b] = pairs of inputs [b << cntShift, (b + 1) << cntShift) under the tap): the sixteen
+// wavefronts of a workgroup sum the rows of the taps up to their own, one row per wavefront at a time, so no pass
+// keeps per-tap totals with device-wide atomics and nothing has to be zeroed before a build.  A workgroup covers
+// `iters` runs of 4096 inputs, which keeps the number of workgroups that repeat these sums small.
 // ---------------------------------------------------------------------------
-__global__ void __launch_bounds__(kRbThreads)
-rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int kVol,
-          const uint32_t* staging, const uint32_t* __restrict__ cnt, uint32_t nBlocks,
-          const uint32_t* __restrict__ totals, int32_t* __restrict__ gather, int32_t* __restrict__ scatter,
-          int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* nbr, int64_t nbrRows,
-          const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int mirror, int inPlace,
-          unsigned long long* __restrict__ masks, uint32_t* fillState, int incrementalFill, int skipIndex) {
-  __shared__ uint32_t scratch[2 * kRbThreads / 64];
+constexpr int kCompactThreads = 1024;
+constexpr int kCompactWaves = kCompactThreads / 64;
+
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (no LDS traffic, no index registers):
+// four shifts inside each row of 16 lanes, then the total of row 0 (2) is added to row 1 (3), then that of rows
+// 0-1 to rows 2-3.
+__device__ __forceinline__ uint32_t waveInclusiveScan(uint32_t v) {
+  v += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x111, 0xF, 0xF, false));  // row_shr:1
+  v += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x112, 0xF, 0xF, false));  // row_shr:2
+  v += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x114, 0xF, 0xF, false));  // row_shr:4
+  v += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x118, 0xF, 0xF, false));  // row_shr:8
+  v += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x142, 0xA, 0xF, false));  // row_bcast:15
+  v += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x143, 0xC, 0xF, false));  // row_bcast:31
+  return v;
+}
+
+// Sum over the 64 lanes, the same value in every lane.
+__device__ __forceinline__ uint32_t waveSum(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(waveInclusiveScan(v)), 63));
+}
+
+__device__ __forceinline__ uint32_t alignSegment(uint32_t v) {
+  return (v + (kSegment - 1)) & ~static_cast<uint32_t>(kSegment - 1);
+}
+
+// Sum of the eight 16-bit counts of `v` whose block index (b0 .. b0 + 7) lies below `limit`.
+__device__ __forceinline__ uint32_t countsBelow(const uint4& v, uint32_t b0, uint32_t limit) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  uint32_t sum = 0;
+  if (b0 + 8 <= limit) {  // the common case: all eight (sad_u16 against 0 adds both halves of a word)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sum = __builtin_amdgcn_sad_u16(w[j], 0u, sum);
+    return sum;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (b0 + 2 * j < limit) sum += w[j] & 0xFFFFu;
+    if (b0 + 2 * j + 1 < limit) sum += w[j] >> 16;
+  }
+  return sum;
+}
+
+// MIRROR: the table is that of a SubM rulebook with "same" padding (see below).  SKIP: the index tensor is left
+// unwritten (nothing reads it): what remains is numIndex and, where inputs were not in rank order, the ranks in
+// the mirrored table turned into rows.  SHIFT: log2 of the inputs per entry of cnt (8, 9 or 10); a wavefront
+// compacts exactly one such block, 1 << (SHIFT - 6) consecutive inputs per lane, so its write position is the
+// workgroup's plus the counts of the workgroup's earlier blocks - after the one barrier behind the sums the
+// wavefronts run on their own, each as soon as its own staging entries have arrived.
+template <bool MIRROR, bool SKIP, int SHIFT>
+__global__ void __launch_bounds__(kCompactThreads) __attribute__((amdgpu_waves_per_eu(8, 8)))
+rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int kVol, const uint32_t* staging,
+          const RbCount* __restrict__ cnt, uint32_t cntPitch, int32_t* __restrict__ gather,
+          int32_t* __restrict__ scatter, int32_t* __restrict__ tapRow, int32_t* numIndex, int32_t* nbr, int64_t nbrRows,
+          const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int inPlace,
+          unsigned long long* __restrict__ masks, uint32_t* fillState, int incrementalFill) {
+  constexpr int ITEMS = 1 << (SHIFT - 6);           // consecutive inputs per lane
+  constexpr int RUN = kCompactThreads * ITEMS;      // inputs per workgroup
+  extern __shared__ uint32_t tapTotal[];           // [kVol] pairs per tap (the taps this workgroup needs)
+  __shared__ uint32_t partBefore;                   // pairs of this tap in the blocks before this workgroup's
   const int tap = blockIdx.y;
-  const uint32_t b = blockIdx.x;
-  if (b == 0 && tap == 0) {  // workgroup-uniform
-    uint32_t part = 0;
-    for (int t = threadIdx.x; t < kVol; t += blockDim.x) part += tapSegment(totals, t);
-    const uint32_t end = blockSum(part, scratch);
-    if (threadIdx.x == 0) {
-      *numIndex = static_cast<int32_t>(end);
-      if (fillState) fillState[1] = end;  // what this pass uses of the index tensor: the next pass clears from here
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = liveCount(numActIn, cap);
+  const int64_t run0 = static_cast<int64_t>(blockIdx.x) * RUN;
+  const int64_t first = run0 + tid * ITEMS;
+  const bool lastTap = tap == kVol - 1;
+  const bool lastSpan = blockIdx.x == gridDim.x - 1;
+  const bool shuffled = perm && *permShuffled;
+
+  if (SKIP) {
+    if (MIRROR && inPlace && shuffled) {
+#pragma unroll
+      for (int q = 0; q < ITEMS / 4; ++q) {
+        if (first + 4 * q >= n) break;
+        uint4* cell = reinterpret_cast<uint4*>(const_cast<uint32_t*>(staging) + static_cast<int64_t>(tap) * pitch + first) + q;
+        uint4 v = *cell;
+        if (v.x != kNone) v.x = perm[v.x];
+        if (v.y != kNone) v.y = perm[v.y];
+        if (v.z != kNone) v.z = perm[v.z];
+        if (v.w != kNone) v.w = perm[v.w];
+        *cell = v;
+      }
+    }
+    if (blockIdx.x != 0 || tap != 0) return;  // workgroup-uniform
+  }
+
+  // the staging entries first: their latency (HBM) covers that of the sums below (L2)
+  uint4 s4[ITEMS / 4];
+#pragma unroll
+  for (int q = 0; q < ITEMS / 4; ++q) {
+    s4[q] = make_uint4(kNone, kNone, kNone, kNone);
+    if (!SKIP && first + 4 * q < n)
+      s4[q] = *(reinterpret_cast<const uint4*>(staging + static_cast<int64_t>(tap) * pitch + first) + q);
+  }
+
+  // ---- pairs per tap (rows of cnt), pairs of this tap before this workgroup's blocks ----
+  const uint32_t liveBlocks = static_cast<uint32_t>((static_cast<int64_t>(n) + (1 << SHIFT) - 1) >> SHIFT);
+  uint32_t firstBlock = blockIdx.x * kCompactWaves;
+  if (firstBlock > liveBlocks) firstBlock = liveBlocks;
+  // pairs of this tap in the workgroup's blocks before this wavefront's: read now, summed behind the barrier
+  uint32_t earlier = 0;
+  if (!SKIP && lane < wave && blockIdx.x * kCompactWaves + lane < liveBlocks)
+    earlier = cnt[static_cast<size_t>(tap) * cntPitch + blockIdx.x * kCompactWaves + lane];
+  // workgroups of the last tap also need that tap's total (the end of the used part of the tensor); the one
+  // workgroup of a build that leaves the tensor unwritten needs every tap's
+  const bool wantAll = SKIP || lastTap;
+  const int lastRow = wantAll ? kVol - 1 : tap;
+  // a wavefront sums rows wave, wave + 16, ..., two rows at a time with the loads of both in flight together
+  // (three loads cover 1536 blocks of a row)
+  for (int row0 = wave; row0 <= lastRow; row0 += 2 * kCompactWaves) {
+    const int row1 = row0 + kCompactWaves;
+    const uint32_t limit0 = (row0 < tap || wantAll) ? liveBlocks : firstBlock;
+    const uint32_t limit1 = row1 > lastRow ? 0u : ((row1 < tap || wantAll) ? liveBlocks : firstBlock);
+    const RbCount* __restrict__ r0 = cnt + static_cast<size_t>(row0) * cntPitch;
+    const RbCount* __restrict__ r1 = cnt + static_cast<size_t>(row1) * cntPitch;
+    uint32_t full0 = 0, full1 = 0, part = 0;
+    for (uint32_t base = 0; base < liveBlocks; base += 3 * 512) {
+      uint4 a[3], b[3];
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        const uint32_t b0 = base + static_cast<uint32_t>(k * 64 + lane) * 8;
+        a[k] = make_uint4(0, 0, 0, 0);
+        b[k] = make_uint4(0, 0, 0, 0);
+        if (b0 < limit0) a[k] = *reinterpret_cast<const uint4*>(r0 + b0);
+        if (b0 < limit1) b[k] = *reinterpret_cast<const uint4*>(r1 + b0);
+      }
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        const uint32_t b0 = base + static_cast<uint32_t>(k * 64 + lane) * 8;
+        full0 += countsBelow(a[k], b0, limit0);
+        full1 += countsBelow(b[k], b0, limit1);
+        if (row0 == tap) part += countsBelow(a[k], b0, firstBlock);
+        if (row1 == tap) part += countsBelow(b[k], b0, firstBlock);
+      }
+    }
+    full0 = waveSum(full0);
+    full1 = waveSum(full1);
+    if (row0 == tap || row1 == tap) part = waveSum(part);
+    if (lane == 0) {
+      tapTotal[row0] = full0;
+      if (row1 <= lastRow) tapTotal[row1] = full1;
+      if (row0 == tap || row1 == tap) partBefore = part;
     }
   }
-  if (skipIndex) {
-    // Nobody reads the index tensor and the probe pass has written table and masks: what is left is turning ranks
-    // into rows where the inputs were not in rank order (in place, in the rows of the mirrored table).
-    if (!(mirror && inPlace && perm && *permShuffled)) return;  // grid-uniform
-    const int64_t at = static_cast<int64_t>(b) * kRbChunk + threadIdx.x * kRbItems;
-    if (at >= liveCount(numActIn, cap)) return;
-    uint4* cell = reinterpret_cast<uint4*>(const_cast<uint32_t*>(staging) + static_cast<int64_t>(tap) * pitch + at);
-    uint4 v = *cell;
-    if (v.x != kNone) v.x = perm[v.x];
-    if (v.y != kNone) v.y = perm[v.y];
-    if (v.z != kNone) v.z = perm[v.z];
-    if (v.w != kNone) v.w = perm[v.w];
-    *cell = v;
+  __syncthreads();
+  uint32_t segs = 0;  // segments of the earlier taps
+  for (int t = lane; t < tap; t += 64) segs += alignSegment(tapTotal[t]);
+  const uint32_t segStart = waveSum(segs);
+  uint32_t end = 0;   // end of the used part of the index tensor (workgroups that summed every row)
+  if (wantAll) {
+    uint32_t all = 0;
+    for (int t = lane; t < kVol; t += 64) all += alignSegment(tapTotal[t]);
+    end = waveSum(all);
+  }
+  if (SKIP) {
+    if (tid == 0) {
+      *numIndex = static_cast<int32_t>(end);
+      if (fillState) fillState[1] = end;
+    }
     return;
   }
-  // The index tensor still holds the previous pass (of this operator, at this address): instead of clearing it at
-  // capacity, write -1 where that pass had entries and this one has none - behind the new end up to the old one,
-  // and in the gap that rounds this tap's segment up to 128.  Only the first workgroups of every tap take part
-  // (at least 64 of them when the grid has as many), so the others do not wait for the segment ends; the range
-  // behind the new end is short unless the scene changed a lot between the two passes.
-  const uint32_t fillers = 64u / static_cast<uint32_t>(kVol) + 1u < gridDim.x ? 64u / static_cast<uint32_t>(kVol) + 1u : gridDim.x;
-  if (incrementalFill && b < fillers) {
-    uint32_t mineBefore = 0, mineAll = 0;
-    for (int t = threadIdx.x; t < kVol; t += blockDim.x) {
-      const uint32_t seg = tapSegment(totals, t);
-      mineAll += seg;
-      if (t < tap) mineBefore += seg;
+  const uint32_t at0 = segStart + partBefore + waveSum(earlier);  // where this wavefront's first pair goes
+
+  // ---- rank of this lane's pairs among the wavefront's ----
+  uint32_t v[ITEMS];
+#pragma unroll
+  for (int q = 0; q < ITEMS / 4; ++q) {
+    v[4 * q] = s4[q].x;
+    v[4 * q + 1] = s4[q].y;
+    v[4 * q + 2] = s4[q].z;
+    v[4 * q + 3] = s4[q].w;
+  }
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    if (first + j >= n) v[j] = kNone;
+    mine += (v[j] != kNone);
+  }
+  const uint32_t incl = waveInclusiveScan(mine);
+  uint32_t at = at0 + incl - mine;
+
+  // Mirror mode (SubM with "same" padding): the pair (tap, in i -> out o) has the twin (kVol-1-tap, in o -> out i),
+  // so row i of the neighbour table under the mirrored tap is simply o - this thread's own staging entry.  The
+  // table is then written here in whole coalesced rows, -1 included: no fill pass, no scatter.  With inPlace the
+  // probe pass already used the table rows as its staging rows (staging + tap * pitch IS the row below): only
+  // what the probe did not leave right is stored - entries of rows past the live count, and rows where ranks have
+  // to become row numbers.
+  int32_t* nbrRow = (MIRROR && nbr) ? nbr + static_cast<int64_t>(kVol - 1 - tap) * nbrRows : nullptr;
+  auto mirrorStore = [&](const uint32_t (&o)[ITEMS]) {
+    if (!nbrRow) return;
+    if (first + ITEMS <= nbrRows && ((reinterpret_cast<uintptr_t>(nbrRow + first) & 15) == 0)) {
+#pragma unroll
+      for (int q = 0; q < ITEMS / 4; ++q)
+        reinterpret_cast<uint4*>(nbrRow + first)[q] = make_uint4(o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < ITEMS; ++j)
+        if (first + j < nbrRows) nbrRow[first + j] = static_cast<int32_t>(o[j]);
     }
-    const uint32_t end = blockSum(mineAll, scratch);
-    const uint32_t myStart = blockSum(mineBefore, scratch);
+  };
+  if (shuffled) {  // block-map SubM: the probe stored ranks; rows are perm[rank]
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j)
+      if (v[j] != kNone) v[j] = perm[v[j]];
+  }
+  if (!inPlace || shuffled || first + ITEMS > n) mirrorStore(v);
+  if (masks && MIRROR && kVol <= 64) {
+    // tile masks of the convolution (bit t of masks[r / 64]: some output row of 64-row tile r / 64 has tap t).
+    // Mirrored table: this thread's consecutive INPUT rows are output rows under tap kVol-1-tap; kTileLanes
+    // lanes cover exactly one tile.
+    constexpr int kTileLanes = 64 / ITEMS;
+    const unsigned long long any = __ballot(mine != 0);
+    if ((lane & (kTileLanes - 1)) == 0 && ((any >> lane) & ((1ull << kTileLanes) - 1ull)) && first < nbrRows)
+      atomicOr(&masks[first >> 6], 1ull << (kVol - 1 - tap));
+  }
+  if constexpr (ITEMS <= 8) {
+    // The wavefront's pairs are packed in LDS first (a lane's pairs start at its exclusive rank) and stored from
+    // there: lane l writes pairs l, l + 64, ... of the wavefront, so every store instruction covers 256
+    // consecutive bytes of a row instead of 64 runs of a few entries.  The buffer is the wavefront's own: LDS
+    // accesses of one wavefront are performed in order, no workgroup barrier is involved.
+    __shared__ uint2 packed[kCompactWaves][64 * ITEMS];
+    uint32_t slot = incl - mine;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      if (v[j] != kNone) {
+        packed[wave][slot++] = make_uint2(static_cast<uint32_t>(first + j), v[j]);
+        // the same pair in output-major form, for the convolution: nbr[tap][output row] = input row
+        if (nbr && !MIRROR && v[j] < static_cast<uint64_t>(nbrRows))
+          nbr[static_cast<int64_t>(tap) * nbrRows + v[j]] = static_cast<int32_t>(first + j);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const uint32_t pairs = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), 63));
+    for (uint32_t k = lane; k < pairs; k += 64) {
+      const uint2 e = packed[wave][k];
+      gather[at0 + k] = static_cast<int32_t>(e.x);
+      scatter[at0 + k] = static_cast<int32_t>(e.y);
+      tapRow[at0 + k] = tap;
+    }
+    (void)at;
+  } else {
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      if (v[j] != kNone) {
+        gather[at] = static_cast<int32_t>(first + j);
+        scatter[at] = static_cast<int32_t>(v[j]);
+        tapRow[at] = tap;
+        ++at;
+        if (nbr && !MIRROR && v[j] < static_cast<uint64_t>(nbrRows))
+          nbr[static_cast<int64_t>(tap) * nbrRows + v[j]] = static_cast<int32_t>(first + j);
+      }
+    }
+  }
+  if (lastTap && lastSpan && tid == 0) {
+    *numIndex = static_cast<int32_t>(end);
+    if (fillState) fillState[1] = end;  // what this pass uses of the index tensor: the next pass clears from here
+  }
+  // The index tensor still holds the previous pass (of this operator, at this address): instead of clearing it at
+  // capacity, write -1 where that pass had entries and this one has none - in the gap that rounds this tap's
+  // segment up to 128 (the wavefront that holds the tap's last pairs), and behind the new end up to the old one
+  // (the workgroups of the last tap, which know the new end; short unless the scene changed a lot).
+  if (!incrementalFill) return;
+  if (lastSpan && wave == kCompactWaves - 1) {
+    const uint32_t pairsEnd = at0 + static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), 63));
+    const uint32_t segEnd = alignSegment(pairsEnd);
+    for (uint32_t i = pairsEnd + lane; i < segEnd; i += 64) {
+      gather[i] = -1;
+      scatter[i] = -1;
+      tapRow[i] = -1;
+    }
+  }
+  if (lastTap) {
     const uint32_t oldEnd = fillState[0];
-    const uint32_t gid = (static_cast<uint32_t>(tap) * fillers + b) * kRbThreads + threadIdx.x;
-    const uint32_t nThreads = fillers * gridDim.y * kRbThreads;
+    const uint32_t gid = blockIdx.x * kCompactThreads + tid, nThreads = gridDim.x * kCompactThreads;
     // segment ends are multiples of 128 entries: 16-byte stores when the three rows are 16-byte aligned
     if (((reinterpret_cast<uintptr_t>(gather) | reinterpret_cast<uintptr_t>(scatter) |
           reinterpret_cast<uintptr_t>(tapRow)) & 15) == 0) {
@@ -584,86 +816,6 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
         scatter[i] = -1;
         tapRow[i] = -1;
       }
-    }
-    if (b == 0 && threadIdx.x < kSegment) {
-      const uint32_t i = myStart + tapPairs(totals, tap) + threadIdx.x;
-      if (i < myStart + tapSegment(totals, tap)) {
-        gather[i] = -1;
-        scatter[i] = -1;
-        tapRow[i] = -1;
-      }
-    }
-  }
-  const int n = liveCount(numActIn, cap);
-  const int64_t first = static_cast<int64_t>(b) * kRbChunk + threadIdx.x * kRbItems;
-  // Mirror mode (SubM with "same" padding): the pair (tap, in i -> out o) has the twin (kVol-1-tap, in o -> out i),
-  // so row i of the neighbour table under the mirrored tap is simply o - this thread's own staging entry.  The
-  // table is then written here in whole coalesced rows, -1 included: no fill pass, no scatter.  With inPlace the
-  // probe pass already used the table rows as its staging rows (staging + tap * pitch IS the row below): only
-  // what the probe did not leave right is stored - entries of rows past the live count, and rows where ranks have
-  // to become row numbers.
-  int32_t* nbrRow = (mirror && nbr) ? nbr + static_cast<int64_t>(kVol - 1 - tap) * nbrRows : nullptr;
-  auto mirrorStore = [&](const uint32_t (&o)[kRbItems]) {
-    if (!nbrRow) return;
-    if (first + kRbItems <= nbrRows && ((reinterpret_cast<uintptr_t>(nbrRow + first) & 15) == 0)) {
-      *reinterpret_cast<uint4*>(nbrRow + first) = make_uint4(o[0], o[1], o[2], o[3]);
-    } else {
-#pragma unroll
-      for (int j = 0; j < kRbItems; ++j)
-        if (first + j < nbrRows) nbrRow[first + j] = static_cast<int32_t>(o[j]);
-    }
-  };
-  const uint32_t none4[kRbItems] = {kNone, kNone, kNone, kNone};
-  if (static_cast<int64_t>(b) * kRbChunk >= n || cnt[static_cast<size_t>(tap) * nBlocks + b] == 0) {  // workgroup-uniform
-    mirrorStore(none4);
-    return;
-  }
-
-  // the staging entries first: their latency overlaps that of the sums below
-  uint4 s4 = make_uint4(kNone, kNone, kNone, kNone);
-  if (first < n) s4 = *reinterpret_cast<const uint4*>(staging + static_cast<int64_t>(tap) * pitch + first);
-  // write position = segments of the earlier taps + pairs of this tap in earlier chunks: both sums are spread
-  // over the threads and share one reduction (one round of loads instead of a serial walk over the taps)
-  uint32_t before = 0;
-  for (uint32_t q = threadIdx.x; q < b; q += blockDim.x) before += cnt[static_cast<size_t>(tap) * nBlocks + q];
-  for (int t = threadIdx.x; t < tap; t += blockDim.x) before += tapSegment(totals, t);
-
-  uint32_t v[kRbItems] = {s4.x, s4.y, s4.z, s4.w};
-  uint32_t mine = 0;
-#pragma unroll
-  for (int j = 0; j < kRbItems; ++j) {
-    if (first + j >= n) v[j] = kNone;
-    mine += (v[j] != kNone);
-  }
-  uint32_t pos;
-  uint32_t at = blockSumAndScan(before, mine, scratch, &pos);  // one pair of barriers for the sum and the ranks
-  at += pos;
-  const bool shuffled = perm && *permShuffled;
-  if (shuffled) {  // block-map SubM: the probe stored ranks; rows are perm[rank]
-#pragma unroll
-    for (int j = 0; j < kRbItems; ++j)
-      if (v[j] != kNone) v[j] = perm[v[j]];
-  }
-  if (!inPlace || shuffled || first + kRbItems > n) mirrorStore(v);
-  if (masks && mirror && kVol <= 64) {
-    // tile masks of the convolution (bit t of masks[r / 64]: some output row of 64-row tile r / 64 has tap t).
-    // Mirrored table: this thread's 4 consecutive INPUT rows are output rows under tap kVol-1-tap; a 16-lane row
-    // covers exactly one tile.
-    const unsigned long long any = __ballot(mine != 0);
-    const int lane = threadIdx.x & 63;
-    if ((lane & 15) == 0 && ((any >> lane) & 0xFFFFull) && first < nbrRows)
-      atomicOr(&masks[first >> 6], 1ull << (kVol - 1 - tap));
-  }
-#pragma unroll
-  for (int j = 0; j < kRbItems; ++j) {
-    if (v[j] != kNone) {
-      gather[at] = static_cast<int32_t>(first + j);
-      scatter[at] = static_cast<int32_t>(v[j]);
-      tapRow[at] = tap;
-      ++at;
-      // the same pair in output-major form, for the convolution: nbr[tap][output row] = input row
-      if (nbr && !mirror && v[j] < static_cast<uint64_t>(nbrRows))
-        nbr[static_cast<int64_t>(tap) * nbrRows + v[j]] = static_cast<int32_t>(first + j);
     }
   }
 }
@@ -827,6 +979,14 @@ bmMarkCandidates(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const 
     const unsigned long long mask = 1ull << bit;
     if ((__builtin_nontemporal_load(&records[rec].bits) & mask) == 0) atomicOr(&records[rec].bits, mask);
   }
+}
+
+// c ? a : b on values: the operands are made opaque first, so that a choice between two elements of a local array
+// stays a register select instead of becoming a dynamically indexed (memory-resident) array.
+__device__ __forceinline__ uint32_t pick(bool c, uint32_t a, uint32_t b) {
+  asm("" : "+v"(a));
+  asm("" : "+v"(b));
+  return c ? a : b;
 }
 
 constexpr uint32_t kScanGroup = 32;  // workgroups of the scan pass that share one first-level ticket
@@ -996,7 +1156,7 @@ __global__ void __launch_bounds__(kRbThreads)
 bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
         int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
         const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut,
-        uint32_t* __restrict__ staging, uint32_t* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
+        uint32_t* __restrict__ staging, RbCount* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
   const int tap = blockIdx.y;
@@ -1221,13 +1381,13 @@ bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_
 }
 
 // SubM probe / strided resolve, one thread per input (see bmProbe for the per-pair form).
-// cnt is accumulated with atomics (four workgroups share one chunk of 1024 inputs) and must start at zero.
+// cnt takes one entry per (tap, 256 inputs).
 template <bool SUBM, int KSEL>
 __global__ void __launch_bounds__(kRbThreads)
 bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
             int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
             uint32_t* __restrict__ perm, uint32_t* permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
-            uint32_t* cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
+            RbCount* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
             int64_t nFillB, uint32_t fillBlocks, int32_t* __restrict__ outCoors, uint32_t nRecords) {
   extern __shared__ __attribute__((aligned(16))) unsigned char nearSmem[];
   uint4* group = reinterpret_cast<uint4*>(nearSmem);                                   // [8][kRbThreads] records
@@ -1309,73 +1469,80 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
   });
   if (KSEL != 0 && mine) atomicAdd(&ldsCnt[lane], mine);
   __syncthreads();
-  const uint32_t chunk = probeBlock / kRbItems;
-  for (int t = threadIdx.x; t < g.kVol; t += blockDim.x) {
-    const uint32_t v = ldsCnt[t];
-    if (v) {
-      atomicAdd(&cnt[static_cast<size_t>(t) * nBlocks + chunk], v);
-      atomicAdd(&totals[t * kTotalSlots + probeBlock % kTotalSlots], v);
-    }
-  }
+  // this workgroup's 256 inputs are one block of counts: plain stores
+  for (int t = threadIdx.x; t < g.kVol; t += blockDim.x)
+    cnt[static_cast<size_t>(t) * nBlocks + probeBlock] = static_cast<RbCount>(ldsCnt[t]);
 }
 
-// The same pass for the kernel shapes of fixedKernelShape (3-D, dilation 1, strides 1 / 2 / 4, not transposed),
-// with K1 threads per input: thread (i, i1) resolves the K2*K3 taps of kernel position i1 along the outermost
-// dim.  A brick is one level of that dim, so these taps look into the 2x2 bricks of ONE level: 4 record loads and
-// 64 bytes of LDS per thread instead of 12 and 192, three times the threads - the pass is bound by the latency
-// of its dependent accesses, and this is what hides it.  Workgroup roles by block index: first the fill
-// workgroups (-1 over the neighbour table, bandwidth-bound work beside latency-bound work), then
-// K1 * probeBlocks probing workgroups (the K1 of one 256-input block next to each other), then the pass only
-// the compaction waits for (rank -> row permutation, or the output coordinates).
+// The same pass for the kernel shapes of fixedKernelShape (3-D, dilation 1, strides 1 / 2 / 4, not transposed):
+// one thread per input resolves all K1*K2*K3 taps.  A brick is one level of the outermost dim, so the taps of
+// kernel position i1 along that dim look into the 2x2 bricks of ONE level: 4 record loads per position, all
+// K1*4 of them issued before the first is used.  Nothing in the pass is accumulated across workgroups: a
+// workgroup owns 256 consecutive inputs, so the pairs per (tap, 256 inputs) go to `cnt` with plain stores, and a
+// wavefront owns one 64-row tile, so the tile masks do too (device-wide atomics run at a few per nanosecond on
+// this part: the 22 per workgroup of an earlier form of this pass cost more than all its loads and stores).
+// Workgroup roles by block index: first the fill workgroups (-1 over the neighbour table, bandwidth-bound work
+// beside latency-bound work), then the probing workgroups, then the pass only the compaction waits for
+// (rank -> row permutation, or the output coordinates).
+constexpr int kProbeThreads = 256;   // inputs per workgroup of the fixed-shape probe = inputs per entry of its counts
+constexpr int kProbeShift = 8;
+static_assert(1 << kProbeShift == kProbeThreads, "counts per workgroup");
+
 template <bool SUBM, int K1, int K2, int K3>
-__global__ void __launch_bounds__(kRbThreads)
-bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
+__global__ void __launch_bounds__(kProbeThreads)
+bmProbeFixed(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
              int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
              uint32_t* __restrict__ perm, uint32_t* permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
-             uint32_t* cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
+             RbCount* __restrict__ cnt, uint32_t cntPitch, int32_t* fillA, int64_t nFillA, int32_t* fillB,
              int64_t nFillB, uint32_t fillBlocks, uint32_t probeBlocks, int32_t* __restrict__ outCoors,
-             uint32_t nRecords, unsigned long long* __restrict__ maskOut, int fixTail, int32_t* __restrict__ nbrDirect,
-             int64_t nbrRows) {
-  // Besides the staging entries the pass can write what a linked convolution reads, so that a build whose index
-  // tensor nobody reads needs no compaction: maskOut (SubM, staging rows = rows of the mirrored table) takes the
-  // tile masks - a wavefront's 64 inputs are one 64-row tile - and fixTail has the rows between the live count
-  // and the capacity set to -1; nbrDirect (strided) takes the pairs straight into the scattered table
-  // nbrDirect[tap][output row] = input row, filled with -1 by the reset pass; staging may then be null.
-  constexpr int KP = K2 * K3;
-  __shared__ uint4 group[4 * kRbThreads];
-  __shared__ uint32_t ldsCnt[KP];
+             uint32_t nRecords, unsigned long long* __restrict__ maskOut, int64_t nMasks, int fixTail,
+             int32_t* __restrict__ nbrDirect, int64_t nbrRows, uint32_t* fillState, int handOver) {
+  // Besides the staging entries the pass writes what a linked convolution reads: maskOut (SubM, staging rows =
+  // rows of the mirrored table) takes the tile masks - a wavefront's 64 inputs are one 64-row tile - and fixTail
+  // has the rows between the live count and the capacity set to -1; nbrDirect (strided, index tensor unread)
+  // takes the pairs straight into the scattered table nbrDirect[tap][output row] = input row, filled with -1 by
+  // the reset pass; staging may then be null.
+  constexpr int KP = K2 * K3, KV = K1 * KP;
+  static_assert(KV <= 64, "one lane per tap keeps the wavefront's pair counts");
+  __shared__ uint32_t ldsCnt[KV];
   if (blockIdx.x < fillBlocks) {
-    const int64_t tid = static_cast<int64_t>(blockIdx.x) * kRbThreads + threadIdx.x;
-    const int64_t stride = static_cast<int64_t>(fillBlocks) * kRbThreads;
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * kProbeThreads + threadIdx.x;
+    const int64_t stride = static_cast<int64_t>(fillBlocks) * kProbeThreads;
     fillMinusOneRange(fillA, nFillA, tid, stride);
     fillMinusOneRange(fillB, nFillB, tid, stride);
     return;
   }
-  const uint32_t pidx = blockIdx.x - fillBlocks;
-  if (pidx >= probeBlocks * K1) {
-    const uint32_t e = pidx - probeBlocks * K1;
+  const uint32_t probeBlock = blockIdx.x - fillBlocks;
+  if (probeBlock >= probeBlocks) {
+    const uint32_t e = probeBlock - probeBlocks;
     if (SUBM) {
-      permuteRow(g, m, coors, liveCount(numActIn, cap), static_cast<int64_t>(e) * kRbThreads + threadIdx.x, records,
+      permuteRow(g, m, coors, liveCount(numActIn, cap), static_cast<int64_t>(e) * kProbeThreads + threadIdx.x, records,
                  chunkBase, perm, permShuffled);
     } else {
-      emitRecordCoords(g, m, records, chunkBase, nRecords, e * (kRbThreads / 64) + (threadIdx.x >> 6), outCoors,
+      emitRecordCoords(g, m, records, chunkBase, nRecords, e * (kProbeThreads / 64) + (threadIdx.x >> 6), outCoors,
                        maxNumActOut);
     }
     return;
   }
-  const int i1 = static_cast<int>(pidx % K1);
-  const uint32_t probeBlock = pidx / K1;
   const int n = liveCount(numActIn, cap);
-  const int64_t i0 = static_cast<int64_t>(probeBlock) * kRbThreads;
+  const int64_t i0 = static_cast<int64_t>(probeBlock) * kProbeThreads;
   const int64_t i = i0 + threadIdx.x;
-  if (i0 >= n) {  // workgroup-uniform
+  const int lane = threadIdx.x & 63;
+  // a build without a reset pass hands the fill state over itself: the end of what the previous pass used
+  if (handOver && probeBlock == 0 && threadIdx.x == 0 && fillState) fillState[0] = fillState[1];
+  if (maskOut && probeBlock == probeBlocks - 1) {  // the entries past the last tile that a convolution reads with it
+    for (int64_t q = (static_cast<int64_t>(probeBlocks) * kProbeThreads >> 6) + threadIdx.x; q < nMasks; q += kProbeThreads)
+      maskOut[q] = 0ull;
+  }
+  if (i0 >= n) {  // workgroup-uniform: no live input here
     if (fixTail && i < cap) {
 #pragma unroll
-      for (int q = 0; q < KP; ++q) staging[static_cast<int64_t>(i1 * KP + q) * pitch + i] = kNone;
+      for (int q = 0; q < KV; ++q) staging[static_cast<int64_t>(q) * pitch + i] = kNone;
     }
+    if (maskOut && lane == 0 && (i >> 6) < nMasks) maskOut[i >> 6] = 0ull;
     return;
   }
-  if (threadIdx.x < KP) ldsCnt[threadIdx.x] = 0;
+  if (threadIdx.x < KV) ldsCnt[threadIdx.x] = 0;
   // rows below the live count get a staging entry, in the grid or not (fixTail: every row below the capacity)
   const bool inRange = i < n || (fixTail && i < cap);
   bool live = i < n;
@@ -1384,6 +1551,7 @@ bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
     live = false;
     c[0] = c[1] = c[2] = c[3] = c[4] = 0;
   }
+  live = live && c[0] >= 0 && c[0] < g.shape[0] && c[1] == 0;
   // per dim and kernel position: validity, brick, cell inside the brick
   auto along = [&](int dim, int pos, int* brick, uint32_t* part) {
     const int st = g.s[dim];
@@ -1394,77 +1562,73 @@ bmProbePlane(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
     *part = static_cast<uint32_t>(o) & ((1u << m.shift[dim]) - 1);
     return num >= 0 && (num & (st - 1)) == 0 && o < g.shape[dim + 1];
   };
-  int brick1;
-  uint32_t part1;
-  const bool ok1 = along(1, i1, &brick1, &part1) && live && c[0] >= 0 && c[0] < g.shape[0] && c[1] == 0;
-  bool ok2[K2], ok3[K3];
-  int b2[K2], b3[K3];
-  uint32_t part2[K2], part3[K3];
+  bool ok1[K1], ok2[K2], ok3[K3];
+  int b1[K1], b2[K2], b3[K3];
+  uint32_t part1[K1], part2[K2], part3[K3];
+#pragma unroll
+  for (int q = 0; q < K1; ++q) ok1[q] = along(1, q, &b1[q], &part1[q]) && live;
 #pragma unroll
   for (int q = 0; q < K2; ++q) ok2[q] = along(2, q, &b2[q], &part2[q]);
 #pragma unroll
   for (int q = 0; q < K3; ++q) ok3[q] = along(3, q, &b3[q], &part3[q]);
   // lower brick of the 2x2 group per dim: that of the highest kernel position (the lowest cell), clamped to 0
   const int base2 = b2[K2 - 1] > 0 ? b2[K2 - 1] : 0, base3 = b3[K3 - 1] > 0 ? b3[K3 - 1] : 0;
-  const uint32_t rec0 = ((static_cast<uint32_t>(ok1 ? c[0] : 0) * static_cast<uint32_t>(m.nb[0])) *
-                             static_cast<uint32_t>(m.nb[1]) + static_cast<uint32_t>(ok1 ? brick1 : 0)) *
-                            static_cast<uint32_t>(m.nb[2]) * static_cast<uint32_t>(m.nb[3]);
-  uint4 loaded[4];
-  uint32_t base[4];
-  bool present[4];
+  const uint32_t levelRecords = static_cast<uint32_t>(m.nb[2]) * static_cast<uint32_t>(m.nb[3]);
+  const uint32_t inLevel = static_cast<uint32_t>(base2 * m.nb[3] + base3);
+  // the records of every level first (independent loads), then the taps
+  uint32_t lo[K1][4], hi[K1][4], pre[K1][4];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int y = base2 + (e >> 1), x = base3 + (e & 1);
-    present[e] = ok1 && y < m.nb[2] && x < m.nb[3];
-    const uint32_t rec = present[e] ? rec0 + static_cast<uint32_t>(y * m.nb[3] + x) : 0u;
-    loaded[e] = *reinterpret_cast<const uint4*>(records + rec);
-    base[e] = chunkBase[rec / kRbChunk];
-  }
+  for (int q1 = 0; q1 < K1; ++q1) {
+    const uint32_t rec0 = (static_cast<uint32_t>(ok1[q1] ? c[0] : 0) * static_cast<uint32_t>(m.nb[0]) *
+                               static_cast<uint32_t>(m.nb[1]) + static_cast<uint32_t>(ok1[q1] ? b1[q1] : 0)) * levelRecords + inLevel;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    loaded[e].z += base[e];  // in-chunk prefix -> global prefix
-    group[e * kRbThreads + threadIdx.x] = present[e] ? loaded[e] : make_uint4(0, 0, 0, 0);
-  }
-  __syncthreads();  // ldsCnt zeroed
-  uint32_t mine = 0;  // lane t of a wavefront counts the wavefront's pairs of tap i1 * KP + t
-  unsigned long long tileBits = 0;  // wavefront-uniform: (mirrored) taps that some input of the wavefront has
-  const int lane = threadIdx.x & 63;
-#pragma unroll
-  for (int q2 = 0; q2 < K2; ++q2)
-#pragma unroll
-    for (int q3 = 0; q3 < K3; ++q3) {
-      uint32_t row = kNone;
-      if (ok1 && ok2[q2] && ok3[q3]) {
-        const int member = (((b2[q2] - base2) & 1) << 1) | ((b3[q3] - base3) & 1);
-        const uint4 v = group[member * kRbThreads + threadIdx.x];
-        const unsigned long long bits = (static_cast<unsigned long long>(v.y) << 32) | v.x;
-        const uint32_t bit = (((part1 << m.shift[2]) | part2[q2]) << m.shift[3]) | part3[q3];
-        if ((bits >> bit) & 1ull) {
-          const uint32_t rank = v.z + static_cast<uint32_t>(__popcll(bits & ((1ull << bit) - 1ull)));
-          // SubM: a rank past the live rows is a cell of a shared map whose row a truncated strided build dropped
-          if (SUBM ? rank < static_cast<uint32_t>(n) : rank < static_cast<uint32_t>(maxNumActOut)) row = rank;
-        }
-      }
-      const int tap = (i1 * K2 + q2) * K3 + q3;
-      if (nbrDirect && row != kNone && row < static_cast<uint64_t>(nbrRows))
-        nbrDirect[static_cast<int64_t>(tap) * nbrRows + row] = static_cast<int32_t>(i);
-      if (staging && inRange) staging[static_cast<int64_t>(tap) * pitch + i] = row;
-      const uint32_t hits = static_cast<uint32_t>(__popcll(__ballot(row != kNone)));
-      if (lane == q2 * K3 + q3) mine += hits;
-      if (hits) tileBits |= 1ull << ((g.kVol - 1 - tap) & 63);
+    for (int e = 0; e < 4; ++e) {
+      const bool present = ok1[q1] && base2 + (e >> 1) < m.nb[2] && base3 + (e & 1) < m.nb[3];
+      const uint32_t rec = present ? rec0 + static_cast<uint32_t>((e >> 1) * m.nb[3] + (e & 1)) : 0u;
+      const uint4 r = *reinterpret_cast<const uint4*>(records + rec);
+      const uint32_t base = chunkBase[rec / kRbChunk];
+      lo[q1][e] = present ? r.x : 0u;
+      hi[q1][e] = present ? r.y : 0u;
+      pre[q1][e] = r.z + base;  // in-chunk prefix -> global prefix
     }
-  if (maskOut && lane == 0 && tileBits) atomicOr(&maskOut[(i0 + (threadIdx.x & ~63)) >> 6], tileBits);
+  }
+  uint32_t mine = 0;  // lane t of a wavefront counts the wavefront's pairs of tap t
+  unsigned long long tileBits = 0;  // wavefront-uniform: (mirrored) taps that some input of the wavefront has
+  const uint32_t rankLimit = SUBM ? static_cast<uint32_t>(n) : static_cast<uint32_t>(maxNumActOut);
+#pragma unroll
+  for (int q1 = 0; q1 < K1; ++q1)
+#pragma unroll
+    for (int q2 = 0; q2 < K2; ++q2) {
+      // the two records of this brick row
+      const bool up = ((b2[q2] - base2) & 1) != 0;
+      const uint32_t lo0 = pick(up, lo[q1][2], lo[q1][0]), hi0 = pick(up, hi[q1][2], hi[q1][0]), pre0 = pick(up, pre[q1][2], pre[q1][0]);
+      const uint32_t lo1 = pick(up, lo[q1][3], lo[q1][1]), hi1 = pick(up, hi[q1][3], hi[q1][1]), pre1 = pick(up, pre[q1][3], pre[q1][1]);
+#pragma unroll
+      for (int q3 = 0; q3 < K3; ++q3) {
+        const bool right = ((b3[q3] - base3) & 1) != 0;
+        const unsigned long long bits = (static_cast<unsigned long long>(pick(right, hi1, hi0)) << 32) | pick(right, lo1, lo0);
+        const uint32_t prefix = pick(right, pre1, pre0);
+        uint32_t row = kNone;
+        const uint32_t bit = (((part1[q1] << m.shift[2]) | part2[q2]) << m.shift[3]) | part3[q3];
+        if (ok1[q1] && ok2[q2] && ok3[q3] && ((bits >> bit) & 1ull)) {
+          const uint32_t rank = prefix + static_cast<uint32_t>(__popcll(bits & ((1ull << bit) - 1ull)));
+          // SubM: a rank past the live rows is a cell of a shared map whose row a truncated strided build dropped
+          if (rank < rankLimit) row = rank;
+        }
+        const int tap = (q1 * K2 + q2) * K3 + q3;
+        if (nbrDirect && row != kNone && row < static_cast<uint64_t>(nbrRows))
+          nbrDirect[static_cast<int64_t>(tap) * nbrRows + row] = static_cast<int32_t>(i);
+        if (staging && inRange) staging[static_cast<int64_t>(tap) * pitch + i] = row;
+        const uint32_t hits = static_cast<uint32_t>(__popcll(__ballot(row != kNone)));
+        if (lane == tap) mine += hits;
+        if (hits) tileBits |= 1ull << (KV - 1 - tap);
+      }
+    }
+  if (maskOut && lane == 0 && (i >> 6) < nMasks) maskOut[i >> 6] = tileBits;
+  __syncthreads();  // ldsCnt zeroed
   if (mine) atomicAdd(&ldsCnt[lane], mine);
   __syncthreads();
-  const uint32_t chunk = probeBlock / kRbItems;
-  if (threadIdx.x < KP) {
-    const uint32_t v = ldsCnt[threadIdx.x];
-    if (v) {
-      const int tap = i1 * KP + threadIdx.x;
-      atomicAdd(&cnt[static_cast<size_t>(tap) * nBlocks + chunk], v);
-      atomicAdd(&totals[tap * kTotalSlots + probeBlock % kTotalSlots], v);
-    }
-  }
+  if (threadIdx.x < KV) cnt[static_cast<size_t>(threadIdx.x) * cntPitch + probeBlock] = static_cast<RbCount>(ldsCnt[threadIdx.x]);
 }
 
 size_t alignUp(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
@@ -1568,8 +1732,11 @@ RbWorkspace planWith(const RbGeom& g, int64_t cap, bool subM, bool blockMap) {
   }
   w.staging = off;
   off = alignUp(off + static_cast<size_t>(g.kVol) * w.pitch * 4);
-  w.cnt = off;     // [kVol, nBlocks], followed (the counters are cleared as one range) by
-  off = alignUp(off + static_cast<size_t>(g.kVol) * w.nBlocks * 4, 16);
+  // pairs per (tap, block of inputs): rows of cntPitch words, one per 256 inputs (the fixed-shape probe) or per
+  // 1024 (the others, which use the head of each row)
+  w.cntPitch = static_cast<uint32_t>(((cap + kRbThreads - 1) / kRbThreads + 7) / 8 * 8);
+  w.cnt = off;     // RbCount [kVol, cntPitch], followed (the counters are cleared as one range) by
+  off = alignUp(off + static_cast<size_t>(g.kVol) * w.cntPitch * sizeof(RbCount), 16);
   w.totals = off;  // [kVol, kTotalSlots] valid pairs per tap in partial sums, [kVol] owned outputs per tap, "rows not
                    // in rank order" flag, scan ticket, first-level scan tickets
   off = alignUp(off + totalsWords(g.kVol, w.nChunks) * 4);
@@ -1695,7 +1862,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   char* ws = static_cast<char*>(workspace);
   uint32_t* staging = reinterpret_cast<uint32_t*>(ws + w.staging);
   int64_t pitch = w.pitch;
-  auto* cnt = reinterpret_cast<uint32_t*>(ws + w.cnt);
+  auto* cnt = reinterpret_cast<RbCount*>(ws + w.cnt);
   auto* totals = reinterpret_cast<uint32_t*>(ws + w.totals);
   uint32_t* ownTotals = totals + g.kVol * kTotalSlots;
   const int64_t rowLen = static_cast<int64_t>(g.kVol) * (cap + kSegment);
@@ -1736,6 +1903,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   bool nbrFilled = mirror;
   bool skipIndex = false;                     // set below when side.skipIndex can be honoured
   bool directScatter = false;                 // the probe pass writes the scattered table itself
+  bool needReset = true;                      // a reset pass opens the build
+  int cntShift = 10;                          // log2 of the inputs one entry of cnt covers
   unsigned long long* compactMasks = masks;   // null when the probe pass writes the masks itself
   const uint32_t* compactPerm = nullptr;      // block-map SubM: staging holds ranks, rows = perm[rank] when shuffled
   const uint32_t* compactPermFlag = nullptr;
@@ -1774,11 +1943,15 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     int32_t* const resetFill = directScatter ? nbrOut : ((near || skipIndex) ? nullptr : fillIndex);
     const int64_t resetFillN = directScatter ? static_cast<int64_t>(g.kVol) * nbrRows : nIndex;
     const int64_t clearRecords = sharedMap ? 0 : static_cast<int64_t>(w.nRecords);
-    hipLaunchKernelGGL(bmReset, fillGrid(clearRecords + (resetFill ? resetFillN / 4 : 0) + 1), block, 0,
-                       stream, reinterpret_cast<uint4*>(records), clearRecords,
-                       resetFill, resetFillN, cnt,
-                       static_cast<int64_t>((w.totals - w.cnt) / 4 + totalsWords(g.kVol, w.nChunks)),
-                       numIndex, masks, nMasks, fillState);
+    // A build on a shared map with the fixed-shape probe leaves nothing to zero: the probe writes counts and tile
+    // masks with plain stores, the compaction sums the counts itself, numIndex is written last.
+    needReset = !(sharedMap && near && ksel != 0 && !directScatter && !resetFill && compactMasks == nullptr);
+    if (needReset)
+      hipLaunchKernelGGL(bmReset, fillGrid(clearRecords + (resetFill ? resetFillN / 4 : 0) + 1), block, 0,
+                         stream, reinterpret_cast<uint4*>(records), clearRecords,
+                         resetFill, resetFillN, reinterpret_cast<uint32_t*>(cnt),
+                         static_cast<int64_t>((w.totals - w.cnt) / 4 + totalsWords(g.kVol, w.nChunks)),
+                         numIndex, masks, nMasks, fillState);
     if (sharedMap) {
       // the strided build that wrote these coordinates marked and scanned this very grid
     } else if (subM) {
@@ -1821,19 +1994,25 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       nbrFilled = true;
 #define D3D_LAUNCH_PROBE_NEAR(SUBM, KSEL)                                                                          \
   hipLaunchKernelGGL((bmProbeNear<SUBM, KSEL>), fused, block, nearLds, stream, g, m, coors, numActIn, cap, pitch,   \
-                     records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals, fillIndex, \
+                     records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.cntPitch, nullptr, fillIndex, \
                      nIndex, fillB, nFillB, quads, outCoors, w.nRecords)
       // fixed kernel shapes: K1 threads per input; fill workgroups only for what there is to fill
       const int64_t fillItems = (probeFillIndex ? nIndex : 0) + nFillB;
       uint32_t planeFill = static_cast<uint32_t>((fillItems / 4 + kRbThreads - 1) / kRbThreads);
       if (planeFill > 1024) planeFill = 1024;
+      // the fixed-shape probe runs workgroups of kProbeThreads inputs
+      const uint32_t fixedBlocks = static_cast<uint32_t>((cap + kProbeThreads - 1) / kProbeThreads > 0 ? (cap + kProbeThreads - 1) / kProbeThreads : 1);
+      const uint32_t fixedExtra = sharedMap ? 0u : (subM ? fixedBlocks : (w.nRecords + kProbeThreads / 64 - 1) / (kProbeThreads / 64));
+      planeFill = (planeFill * kRbThreads + kProbeThreads - 1) / kProbeThreads;
 #define D3D_LAUNCH_PROBE_PLANE(SUBM, K1, K2, K3)                                                                    \
-  hipLaunchKernelGGL((bmProbePlane<SUBM, K1, K2, K3>), dim3(planeFill + probeBlocks * K1 + extra), block, 0, stream, \
+  hipLaunchKernelGGL((bmProbeFixed<SUBM, K1, K2, K3>), dim3(planeFill + fixedBlocks + fixedExtra), dim3(kProbeThreads), 0, stream, \
                      g, m, coors, numActIn, cap, pitch, records, chunkBase, perm, permShuffled, maxNumActOut,     \
-                     (directScatter && skipIndex) ? nullptr : staging, cnt, w.nBlocks, totals, probeFillIndex,      \
+                     (directScatter && skipIndex) ? nullptr : staging, cnt, w.cntPitch, probeFillIndex,             \
                      nIndex, fillB, nFillB, planeFill,                                                               \
-                     probeBlocks, outCoors, w.nRecords, probeMasks ? masks : nullptr, (skipIndex && subM) ? 1 : 0,   \
-                     directScatter ? nbrOut : nullptr, nbrRows)
+                     fixedBlocks, outCoors, w.nRecords, probeMasks ? masks : nullptr, nMasks,                        \
+                     (subM && inPlace) ? 1 : 0, directScatter ? nbrOut : nullptr, nbrRows, fillState,               \
+                     needReset ? 0 : 1)
+      cntShift = ksel != 0 ? kProbeShift : 8;  // the one-thread-per-input probes count per workgroup
       if (subM) {
         switch (ksel) {
           case 1: D3D_LAUNCH_PROBE_PLANE(true, 3, 3, 3); break;
@@ -1855,10 +2034,10 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
 #undef D3D_LAUNCH_PROBE_NEAR
     } else if (subM) {
       hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, pitch, records, chunkBase, perm,
-                         permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
+                         permShuffled, maxNumActOut, staging, cnt, w.cntPitch, nullptr);
     } else {
       hipLaunchKernelGGL(bmProbe<false>, perTap, block, 0, stream, g, m, coors, numActIn, cap, pitch, records, chunkBase, perm,
-                         permShuffled, maxNumActOut, staging, cnt, w.nBlocks, totals);
+                         permShuffled, maxNumActOut, staging, cnt, w.cntPitch, nullptr);
     }
   } else {
     auto* table = reinterpret_cast<unsigned long long*>(ws + w.table);
@@ -1872,7 +2051,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     if (subM) {
       hipLaunchKernelGGL(rbSubmInsert, perInput, block, 0, stream, g, coors, numActIn, cap, table, mask);
       hipLaunchKernelGGL(rbSubmProbe, perTap, block, 0, stream, g, coors, numActIn, cap, pitch, table, mask,
-                         staging, cnt, w.nBlocks, totals);
+                         staging, cnt, w.cntPitch, nullptr);
     } else {
       hipLaunchKernelGGL(rbConvInsert, perTap, block, 0, stream, g, coors, numActIn, cap, pitch, table, mask,
                          staging);
@@ -1881,7 +2060,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       hipLaunchKernelGGL(rbConvAssign, perTap, block, 0, stream, g, numActIn, cap, pitch, table, staging, ownCnt,
                          w.nBlocks, ownTotals, ids, outCoors, numActOut, maxNumActOut);
       hipLaunchKernelGGL(rbConvResolve, perTap, block, 0, stream, numActIn, cap, pitch, ids, staging, maxNumActOut,
-                         cnt, w.nBlocks, totals);
+                         cnt, w.cntPitch, nullptr);
     }
   }
   if (nbrOut && nbrRows > 0 && !nbrFilled)
@@ -1889,12 +2068,29 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
                        static_cast<int64_t>(g.kVol) * nbrRows);
   // with the index tensor unwritten only a build that may have to turn ranks into rows needs the whole grid; the
   // others launch the one workgroup that writes numIndex
-  const dim3 compactGrid = (skipIndex && !compactPerm) ? dim3(1, 1) : perTap;
-  hipLaunchKernelGGL(rbCompact, compactGrid, block, 0, stream, numActIn, cap, pitch, g.kVol, staging, cnt, w.nBlocks,
-                     totals, index, index + rowLen, index + 2 * rowLen, numIndex,
-                     (nbrRows > 0 && !directScatter) ? nbrOut : nullptr, nbrRows,
-                     compactPerm, compactPermFlag, mirror ? 1 : 0, inPlace ? 1 : 0, compactMasks, fillState,
-                     incremental ? 1 : 0, skipIndex ? 1 : 0);
+  const int64_t compactRun = static_cast<int64_t>(kCompactWaves) << cntShift;  // a wavefront per block of counts
+  const dim3 allSpans(static_cast<unsigned>((cap + compactRun - 1) / compactRun > 0 ? (cap + compactRun - 1) / compactRun : 1),
+                      g.kVol);
+  const dim3 compactGrid = (skipIndex && !compactPerm) ? dim3(1, 1) : allSpans;
+#define D3D_LAUNCH_COMPACT(MIRROR, SKIP, SHIFT)                                                                       \
+  hipLaunchKernelGGL((rbCompact<MIRROR, SKIP, SHIFT>), compactGrid, dim3(kCompactThreads),                            \
+                     static_cast<size_t>(g.kVol) * 4, stream, numActIn, cap, pitch, g.kVol, staging, cnt, w.cntPitch,  \
+                     index, index + rowLen, index + 2 * rowLen, numIndex,                                             \
+                     (nbrRows > 0 && !directScatter) ? nbrOut : nullptr, nbrRows, compactPerm, compactPermFlag,        \
+                     inPlace ? 1 : 0, compactMasks, fillState, incremental ? 1 : 0)
+#define D3D_LAUNCH_COMPACT_SHIFT(MIRROR, SKIP)                        \
+  do {                                                                \
+    if (cntShift == 8) D3D_LAUNCH_COMPACT(MIRROR, SKIP, 8);           \
+    else if (cntShift == 9) D3D_LAUNCH_COMPACT(MIRROR, SKIP, 9);      \
+    else D3D_LAUNCH_COMPACT(MIRROR, SKIP, 10);                        \
+  } while (0)
+  if (skipIndex) {
+    if (mirror) D3D_LAUNCH_COMPACT_SHIFT(true, true); else D3D_LAUNCH_COMPACT_SHIFT(false, true);
+  } else {
+    if (mirror) D3D_LAUNCH_COMPACT_SHIFT(true, false); else D3D_LAUNCH_COMPACT_SHIFT(false, false);
+  }
+#undef D3D_LAUNCH_COMPACT_SHIFT
+#undef D3D_LAUNCH_COMPACT
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;
 }
