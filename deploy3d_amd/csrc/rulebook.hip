@@ -611,15 +611,6 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
     if (blockIdx.x != 0 || tap != 0) return;  // workgroup-uniform
   }
 
-  // the staging entries first: their latency (HBM) covers that of the sums below (L2)
-  uint4 s4[ITEMS / 4];
-#pragma unroll
-  for (int q = 0; q < ITEMS / 4; ++q) {
-    s4[q] = make_uint4(kNone, kNone, kNone, kNone);
-    if (!SKIP && first + 4 * q < n)
-      s4[q] = *(reinterpret_cast<const uint4*>(staging + static_cast<int64_t>(tap) * pitch + first) + q);
-  }
-
   // ---- pairs per tap (rows of cnt), pairs of this tap before this workgroup's blocks ----
   const uint32_t liveBlocks = static_cast<uint32_t>((static_cast<int64_t>(n) + (1 << SHIFT) - 1) >> SHIFT);
   uint32_t firstBlock = blockIdx.x * kCompactWaves;
@@ -632,42 +623,76 @@ rbCompact(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, int 
   // workgroup of a build that leaves the tensor unwritten needs every tap's
   const bool wantAll = SKIP || lastTap;
   const int lastRow = wantAll ? kVol - 1 : tap;
-  // a wavefront sums rows wave, wave + 16, ..., two rows at a time with the loads of both in flight together
-  // (three loads cover 1536 blocks of a row)
-  for (int row0 = wave; row0 <= lastRow; row0 += 2 * kCompactWaves) {
+  // A wavefront sums rows wave, wave + 16, ..., two rows at a time with the loads of both in flight together
+  // (three loads cover 1536 blocks of a row).  Loads return in the order of their issue: the rows (L2) are
+  // requested before the staging entries (HBM), so that the sums do not wait for those.
+  auto rowLimit = [&](int row) -> uint32_t {
+    return row > lastRow ? 0u : ((row < tap || wantAll) ? liveBlocks : firstBlock);
+  };
+  auto loadRows = [&](int row0, uint32_t base, uint4 (&a)[3], uint4 (&b)[3]) {
     const int row1 = row0 + kCompactWaves;
-    const uint32_t limit0 = (row0 < tap || wantAll) ? liveBlocks : firstBlock;
-    const uint32_t limit1 = row1 > lastRow ? 0u : ((row1 < tap || wantAll) ? liveBlocks : firstBlock);
-    const RbCount* __restrict__ r0 = cnt + static_cast<size_t>(row0) * cntPitch;
-    const RbCount* __restrict__ r1 = cnt + static_cast<size_t>(row1) * cntPitch;
-    uint32_t full0 = 0, full1 = 0, part = 0;
-    for (uint32_t base = 0; base < liveBlocks; base += 3 * 512) {
-      uint4 a[3], b[3];
+    const uint32_t limit0 = rowLimit(row0), limit1 = rowLimit(row1);
 #pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        const uint32_t b0 = base + static_cast<uint32_t>(k * 64 + lane) * 8;
-        a[k] = make_uint4(0, 0, 0, 0);
-        b[k] = make_uint4(0, 0, 0, 0);
-        if (b0 < limit0) a[k] = *reinterpret_cast<const uint4*>(r0 + b0);
-        if (b0 < limit1) b[k] = *reinterpret_cast<const uint4*>(r1 + b0);
-      }
-#pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        const uint32_t b0 = base + static_cast<uint32_t>(k * 64 + lane) * 8;
-        full0 += countsBelow(a[k], b0, limit0);
-        full1 += countsBelow(b[k], b0, limit1);
-        if (row0 == tap) part += countsBelow(a[k], b0, firstBlock);
-        if (row1 == tap) part += countsBelow(b[k], b0, firstBlock);
-      }
+    for (int k = 0; k < 3; ++k) {
+      const uint32_t b0 = base + static_cast<uint32_t>(k * 64 + lane) * 8;
+      a[k] = make_uint4(0, 0, 0, 0);
+      b[k] = make_uint4(0, 0, 0, 0);
+      if (b0 < limit0) a[k] = *reinterpret_cast<const uint4*>(cnt + static_cast<size_t>(row0) * cntPitch + b0);
+      if (b0 < limit1) b[k] = *reinterpret_cast<const uint4*>(cnt + static_cast<size_t>(row1) * cntPitch + b0);
     }
+  };
+  auto sumRows = [&](int row0, uint32_t base, const uint4 (&a)[3], const uint4 (&b)[3], uint32_t* full0,
+                     uint32_t* full1, uint32_t* part) {
+    const int row1 = row0 + kCompactWaves;
+    const uint32_t limit0 = rowLimit(row0), limit1 = rowLimit(row1);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const uint32_t b0 = base + static_cast<uint32_t>(k * 64 + lane) * 8;
+      *full0 += countsBelow(a[k], b0, limit0);
+      *full1 += countsBelow(b[k], b0, limit1);
+      if (row0 == tap) *part += countsBelow(a[k], b0, firstBlock);
+      if (row1 == tap) *part += countsBelow(b[k], b0, firstBlock);
+    }
+  };
+  auto publishRows = [&](int row0, uint32_t full0, uint32_t full1, uint32_t part) {
+    const int row1 = row0 + kCompactWaves;
     full0 = waveSum(full0);
     full1 = waveSum(full1);
     if (row0 == tap || row1 == tap) part = waveSum(part);
     if (lane == 0) {
-      tapTotal[row0] = full0;
+      if (row0 <= lastRow) tapTotal[row0] = full0;
       if (row1 <= lastRow) tapTotal[row1] = full1;
       if (row0 == tap || row1 == tap) partBefore = part;
     }
+  };
+  uint4 headA[3], headB[3];
+  loadRows(wave, 0, headA, headB);
+  // the staging entries: their latency (HBM) covers the sums below
+  uint4 s4[ITEMS / 4];
+#pragma unroll
+  for (int q = 0; q < ITEMS / 4; ++q) {
+    s4[q] = make_uint4(kNone, kNone, kNone, kNone);
+    if (!SKIP && first + 4 * q < n)
+      s4[q] = *(reinterpret_cast<const uint4*>(staging + static_cast<int64_t>(tap) * pitch + first) + q);
+  }
+  {
+    uint32_t full0 = 0, full1 = 0, part = 0;
+    sumRows(wave, 0, headA, headB, &full0, &full1, &part);
+    for (uint32_t base = 3 * 512; base < liveBlocks; base += 3 * 512) {  // more than 1536 blocks in a row
+      uint4 a[3], b[3];
+      loadRows(wave, base, a, b);
+      sumRows(wave, base, a, b, &full0, &full1, &part);
+    }
+    publishRows(wave, full0, full1, part);
+  }
+  for (int row0 = wave + 2 * kCompactWaves; row0 <= lastRow; row0 += 2 * kCompactWaves) {  // more than 32 taps
+    uint32_t full0 = 0, full1 = 0, part = 0;
+    for (uint32_t base = 0; base < liveBlocks; base += 3 * 512) {
+      uint4 a[3], b[3];
+      loadRows(row0, base, a, b);
+      sumRows(row0, base, a, b, &full0, &full1, &part);
+    }
+    publishRows(row0, full0, full1, part);
   }
   __syncthreads();
   uint32_t segs = 0;  // segments of the earlier taps
@@ -1484,8 +1509,8 @@ bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32
 // Workgroup roles by block index: first the fill workgroups (-1 over the neighbour table, bandwidth-bound work
 // beside latency-bound work), then the probing workgroups, then the pass only the compaction waits for
 // (rank -> row permutation, or the output coordinates).
-constexpr int kProbeThreads = 256;   // inputs per workgroup of the fixed-shape probe = inputs per entry of its counts
-constexpr int kProbeShift = 8;
+constexpr int kProbeThreads = 512;   // inputs per workgroup of the fixed-shape probe = inputs per entry of its counts
+constexpr int kProbeShift = 9;
 static_assert(1 << kProbeShift == kProbeThreads, "counts per workgroup");
 
 template <bool SUBM, int K1, int K2, int K3>

@@ -164,11 +164,16 @@ class SparseBackbone:
         main = side = None
         if self.overlap:
             if self._side is None:  # strided rulebooks feed each other; SubM rulebooks hang off them
-                self._side = {False: torch.cuda.Stream(), True: torch.cuda.Stream()}
+                import os
+                if os.environ.get("D3D_ONE_SIDE"):
+                    one = torch.cuda.Stream()
+                    self._side = {False: one, True: one}
+                else:
+                    self._side = {False: torch.cuda.Stream(), True: torch.cuda.Stream()}
             main, side = torch.cuda.current_stream(), self._side
             fork = torch.cuda.Event()
             fork.record(main)
-            for st in side.values():
+            for st in set(side.values()):
                 st.wait_event(fork)
         rulebooks = {}
         inputs = {}
