@@ -108,7 +108,20 @@ struct RbSide {
   uint32_t* mapChunkBase = nullptr;
   bool useSharedMap = false;
   bool mapWritten = false;              // out: a strided build left its finished map in mapRecords / mapChunkBase
+  // Two maps in turn: with mapState (zeroed when allocated, kept between passes: [0] scans performed so far, [1]
+  // "rows not in rank order", [2] scan ticket, [3..] first-level scan tickets) and mapStride (records from the
+  // first map to the second; mapRecords holds both, zeroed when allocated) a build needs no reset pass: the scan of
+  // one build clears the map the next one marks.  Any build (SubM on its own inputs too) may be given its map
+  // this way.  A SubM build on a shared map passes what the build that wrote it used.
+  uint32_t* mapState = nullptr;
+  int64_t mapStride = 0;
+  bool mapDouble = false;               // out: the build alternated between the two maps (in, with useSharedMap:
+                                        // the build that wrote the shared map did)
+  bool mapDirty = false;                // a build with a reset pass has used these maps: keep the reset pass
 };
+
+// 32-bit words of RbSide::mapState for a map of `chunkBaseBytes` bytes of chunk bases.
+size_t mapStateWords(size_t chunkBaseBytes);
 
 // Bytes of the block map of g's output grid (records, chunk bases); 0 when the grid takes the hash instead.
 void blockMapBytes(const RbGeom& g, int64_t cap, size_t* records, size_t* chunkBase);

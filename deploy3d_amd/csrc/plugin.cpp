@@ -59,6 +59,18 @@ struct DeviceBuffer {
     bytes = n;
     return D3D_OK;
   }
+  // a fresh, zeroed allocation of n bytes, whatever was held before
+  int32_t reallocZeroed(size_t n) {
+    if (ptr) {
+      D3D_HIP_CHECK(hipFree(ptr));
+      ptr = nullptr;
+      bytes = 0;
+    }
+    D3D_HIP_CHECK(hipMalloc(&ptr, n));
+    bytes = n;
+    D3D_HIP_CHECK(hipMemset(ptr, 0, n));
+    return D3D_OK;
+  }
   int32_t upload(const void* src, size_t n) {
     int32_t rc = reserve(n);
     if (rc != D3D_OK) return rc;
@@ -172,6 +184,13 @@ struct RulebookLink {
   // block map of the output grid, kept for the SubM operators that run on this (strided) operator's outputs
   bool shareMap = false;          // some SubM operator is linked to these coordinates
   DeviceBuffer mapRecords, mapChunkBase;
+  // an operator that keeps its map between passes holds two of them (mapStride records apart) and the state
+  // words of RbSide::mapState: its builds then need no reset pass
+  DeviceBuffer mapState;
+  int64_t mapStride = 0;
+  bool mapDouble = false;         // the last build alternated between the two maps
+  bool mapDirty = false;          // a build with a reset pass has used the first map since the allocation: the
+                                  // two no longer alternate cleanly, builds keep their reset pass from then on
   bool mapValid = false;
   const void* mapCoors = nullptr;     // outCoors / numActOut the map belongs to
   const void* mapNumAct = nullptr;
@@ -471,12 +490,34 @@ struct IdxPlugin final : d3d_plugin {
     // outputs, a SubM operator takes the map of the operator that wrote the coordinates it is handed
     std::shared_ptr<RulebookLink> source = subM ? coordSource : nullptr;
     std::unique_lock<std::mutex> sourceLock;
-    if (!subM && link->shareMap && !g_noAlloc) {
+    if (((!subM && link->shareMap) || persistentIndex) && !g_noAlloc) {
+      // The map is kept in memory of this operator: for the SubM operators linked to its outputs, and - two maps
+      // in turn - so that a build needs no reset pass.  Allocated (and zeroed) on first use, or when the grid
+      // grows; never while the stream is being captured.
       size_t recBytes = 0, chunkBytes = 0;
       blockMapBytes(g, cap, &recBytes, &chunkBytes);
-      if (recBytes && link->mapRecords.reserve(recBytes) == D3D_OK && link->mapChunkBase.reserve(chunkBytes) == D3D_OK) {
+      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+      (void)hipStreamIsCapturing(stream, &capturing);
+      const size_t stateBytes = mapStateWords(chunkBytes) * 4;
+      // the two maps alternate cleanly only among builds on one grid size: another size takes a new allocation
+      auto have = [&]() {
+        return link->mapRecords.bytes >= 2 * recBytes && link->mapChunkBase.bytes >= chunkBytes &&
+               link->mapState.bytes >= stateBytes && link->mapStride * 16 == static_cast<int64_t>(recBytes);
+      };
+      if (recBytes && !have() && capturing == hipStreamCaptureStatusNone) {
+        link->mapStride = 0;
+        if (link->mapRecords.reallocZeroed(2 * recBytes) == D3D_OK && link->mapChunkBase.reserve(chunkBytes) == D3D_OK &&
+            link->mapState.reallocZeroed(stateBytes) == D3D_OK) {
+          link->mapStride = static_cast<int64_t>(recBytes / 16);
+          link->mapDirty = false;
+        }
+      }
+      if (recBytes && have()) {
         side.mapRecords = link->mapRecords.ptr;
         side.mapChunkBase = static_cast<uint32_t*>(link->mapChunkBase.ptr);
+        side.mapState = static_cast<uint32_t*>(link->mapState.ptr);
+        side.mapStride = link->mapStride;
+        side.mapDirty = link->mapDirty;
       }
     }
     link->mapValid = false;
@@ -488,6 +529,9 @@ struct IdxPlugin final : d3d_plugin {
       if (same) {
         side.mapRecords = source->mapRecords.ptr;
         side.mapChunkBase = static_cast<uint32_t*>(source->mapChunkBase.ptr);
+        side.mapState = static_cast<uint32_t*>(source->mapState.ptr);
+        side.mapStride = source->mapStride;
+        side.mapDouble = source->mapDouble;
         side.useSharedMap = true;
       }
     }
@@ -510,6 +554,10 @@ struct IdxPlugin final : d3d_plugin {
       if (side.fillState && side.indexWritten) {
         link->primedIndex = outputs[0];
         link->primedRowLen = rowLen;
+      }
+      if (!side.useSharedMap) {
+        link->mapDouble = side.mapDouble;
+        if (side.mapRecords && !side.mapDouble) link->mapDirty = true;
       }
       if (side.mapWritten) {
         link->mapValid = true;

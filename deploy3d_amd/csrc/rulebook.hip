@@ -869,6 +869,21 @@ struct __attribute__((aligned(16))) BmRecord {
   uint32_t pad;
 };
 
+// The records a kernel works on.  A build whose caller keeps the map between passes alternates between two maps
+// (`stride` records apart): `*epoch` counts the scans performed so far, the scan pass of a build clears the
+// occupancy bits of the map the NEXT build will mark and then advances the count, so no pass has to zero a map
+// before marking it.  Kernels before (and including) the scan use bias 0, kernels behind it bias 1 (the count
+// has moved on by then).  epoch == nullptr: one map at `base`, zeroed by a reset pass.
+struct RecRef {
+  BmRecord* base;
+  uint32_t* epoch;
+  uint32_t stride;
+  uint32_t bias;
+  __device__ __forceinline__ BmRecord* get() const {
+    return epoch ? base + static_cast<size_t>((*epoch + bias) & 1u) * stride : base;
+  }
+};
+
 struct BlockMap {
   int shift[kMaxSpatial];  // log2 brick extent per spatial dim (extents multiply to 64)
   int nb[kMaxSpatial];     // bricks per dim
@@ -972,7 +987,11 @@ __device__ __forceinline__ void orRuns(BmRecord* records, uint32_t rec, unsigned
 // SubM: mark the input voxels.
 __global__ void __launch_bounds__(kRbThreads)
 bmMarkInputs(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
-             BmRecord* records) {
+             RecRef recRef, uint32_t* clearFlag) {
+  BmRecord* records = recRef.get();
+  // a build without a reset pass: the "rows not in rank order" flag of the previous pass goes here (the pass that
+  // raises it comes behind the scan)
+  if (clearFlag && blockIdx.x == 0 && threadIdx.x == 0) *clearFlag = 0u;
   const int n = liveCount(numActIn, cap);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   uint32_t rec = kNone, bit = 0;
@@ -987,7 +1006,8 @@ bmMarkInputs(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
 // A bit that a plain read already shows set needs no atomic; bits are only ever set.
 __global__ void __launch_bounds__(kRbThreads)
 bmMarkCandidates(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn,
-                 int64_t cap, BmRecord* records) {
+                 int64_t cap, RecRef recRef) {
+  BmRecord* records = recRef.get();
   const int n = liveCount(numActIn, cap);
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
   if (first >= n) return;
@@ -1021,10 +1041,14 @@ constexpr uint32_t kScanGroup = 32;  // workgroups of the scan pass that share o
 // totals into exclusive chunk bases and writes numActOut = min(total, maxNumActOut) for strided convolutions.
 template <bool ORDERED>
 __global__ void __launch_bounds__(kRbThreads)
-bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, uint32_t nChunks, uint32_t* ticket,
+bmScan(RecRef recRef, uint32_t nRecords, uint32_t* chunkBase, uint32_t nChunks, uint32_t* ticket,
        uint32_t* groupTickets, int32_t* numActOut, int32_t maxNumActOut) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   __shared__ uint32_t isLast;
+  const uint32_t epoch = recRef.epoch ? *recRef.epoch : 0u;
+  BmRecord* __restrict__ records = recRef.base + static_cast<size_t>(epoch & 1u) * (recRef.epoch ? recRef.stride : 0u);
+  // two maps: the occupancy bits of the one the next build marks are cleared here, record by record
+  BmRecord* __restrict__ other = recRef.epoch ? recRef.base + static_cast<size_t>((epoch + 1u) & 1u) * recRef.stride : nullptr;
   // A wavefront takes 256 consecutive records as 4 rows of 64: lane l reads records l, 64 + l, 128 + l, 192 + l of
   // them, so every load instruction covers 1 KB of consecutive memory.  Counts are at most 64 and a row's running
   // sum at most 4096, so two rows share one 32-bit lane scan (16 bits each).
@@ -1033,8 +1057,10 @@ bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, u
   const uint32_t first = blockIdx.x * kRbChunk + wave * 256 + lane;
   uint32_t count[kRbItems];
 #pragma unroll
-  for (int j = 0; j < kRbItems; ++j)
+  for (int j = 0; j < kRbItems; ++j) {
     count[j] = first + j * 64 < nRecords ? static_cast<uint32_t>(__popcll(records[first + j * 64].bits)) : 0u;
+    if (other && first + j * 64 < nRecords) other[first + j * 64].bits = 0ull;
+  }
   uint32_t inclA = count[0] | (count[1] << 16), inclB = count[2] | (count[3] << 16);
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
@@ -1110,20 +1136,28 @@ bmScan(BmRecord* __restrict__ records, uint32_t nRecords, uint32_t* chunkBase, u
   }
   if (threadIdx.x == 0 && numActOut)
     *numActOut = static_cast<int32_t>(running < static_cast<uint32_t>(maxNumActOut) ? running : maxNumActOut);
+  // Every other workgroup has drawn its tickets (and read the scan count before that): the counters go back to
+  // zero for the next pass, and with two maps the count moves on - the passes behind this one see this map as
+  // the finished one, the next build marks the other.
+  if (recRef.epoch) {
+    const uint32_t nGroups = (nChunks + kScanGroup - 1) / kScanGroup;
+    for (uint32_t q = threadIdx.x; q < nGroups; q += blockDim.x) groupTickets[q] = 0u;
+    if (threadIdx.x == 0) {
+      *ticket = 0u;
+      *recRef.epoch = epoch + 1u;
+    }
+  }
 }
 
 
-// Strided convolutions: output coordinates in rank order (reference: coorsOutOrganizeKernel,
-// index.cu:104-121).  One wavefront per record, one lane per cell of the brick.
-// outCoors[rank] = coordinate of every occupied cell of record `rec`; one wavefront per record, lane = cell
-__device__ __forceinline__ void emitRecordCoords(const RbGeom& g, const BlockMap& m, const BmRecord* __restrict__ records,
-                                                 const uint32_t* __restrict__ chunkBase, uint32_t nRecords, uint32_t rec,
-                                                 int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
-  if (rec >= nRecords) return;
-  const BmRecord r = records[rec];
+constexpr uint32_t kEmitGroup = 8;  // records per wavefront of the coordinate pass
+
+// One cell per lane of an occupied record (bits, global prefix of record `rec`): outCoors[rank] = its coordinate.
+__device__ __forceinline__ void emitCells(const RbGeom& g, const BlockMap& m, unsigned long long bits, uint32_t prefix,
+                                          uint32_t rec, int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
   uint32_t bit = threadIdx.x & 63;
-  if (!((r.bits >> bit) & 1ull)) return;
-  const uint32_t id = bmRank(r, bit, chunkBase, rec);
+  if (!((bits >> bit) & 1ull)) return;
+  const uint32_t id = prefix + static_cast<uint32_t>(__popcll(bits & ((1ull << bit) - 1ull)));
   if (id >= static_cast<uint32_t>(maxNumActOut)) return;
   const int pad = kMaxSpatial - g.nd;
   int32_t* row = outCoors + static_cast<size_t>(id) * (g.nd + 1);
@@ -1140,9 +1174,42 @@ __device__ __forceinline__ void emitRecordCoords(const RbGeom& g, const BlockMap
   row[0] = static_cast<int32_t>(q);
 }
 
+// Strided convolutions: output coordinates in rank order (reference: coorsOutOrganizeKernel,
+// index.cu:104-121).  A wavefront takes kEmitGroup consecutive records, one per lane, and then walks the occupied
+// ones among them with one cell per lane: on a sparse grid most records are empty and cost one load between
+// several (a wavefront per 64 records measured 16 -> 41 us on a small dense grid, where every record is a turn of
+// the loop; a wavefront per record 42 -> 36 us on a large sparse one).
+__device__ __forceinline__ void emitRecordCoords(const RbGeom& g, const BlockMap& m, const BmRecord* __restrict__ records,
+                                                 const uint32_t* __restrict__ chunkBase, uint32_t nRecords,
+                                                 uint32_t group, int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
+  const uint32_t rec0 = group * kEmitGroup;
+  if (rec0 >= nRecords) return;  // wavefront-uniform
+  const uint32_t lane = threadIdx.x & 63;
+  uint32_t lo = 0, hi = 0, prefix = 0;
+  if (lane < kEmitGroup && rec0 + lane < nRecords) {
+    const uint4 r = *reinterpret_cast<const uint4*>(records + rec0 + lane);
+    lo = r.x;
+    hi = r.y;
+    prefix = r.z;
+  }
+  unsigned long long occupied = __ballot((lo | hi) != 0u);
+  if (occupied == 0ull) return;
+  prefix += chunkBase[((lane < kEmitGroup && rec0 + lane < nRecords) ? rec0 + lane : rec0) / kRbChunk];
+  while (occupied) {
+    const int r = __builtin_ctzll(occupied);
+    occupied &= occupied - 1ull;
+    const unsigned long long bits =
+        (static_cast<unsigned long long>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), r))) << 32) |
+        static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), r));
+    const uint32_t pre = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(prefix), r));
+    emitCells(g, m, bits, pre, rec0 + static_cast<uint32_t>(r), outCoors, maxNumActOut);
+  }
+}
+
 __global__ void __launch_bounds__(kRbThreads)
-bmEmitCoords(RbGeom g, BlockMap m, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+bmEmitCoords(RbGeom g, BlockMap m, RecRef recRef, const uint32_t* __restrict__ chunkBase,
              uint32_t nRecords, int32_t* __restrict__ outCoors, int32_t maxNumActOut) {
+  const BmRecord* __restrict__ records = recRef.get();
   emitRecordCoords(g, m, records, chunkBase, nRecords, blockIdx.x * (kRbThreads / 64) + (threadIdx.x >> 6), outCoors,
                    maxNumActOut);
 }
@@ -1166,8 +1233,9 @@ __device__ __forceinline__ void permuteRow(const RbGeom& g, const BlockMap& m, c
 
 __global__ void __launch_bounds__(kRbThreads)
 bmPermutation(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn,
-              int64_t cap, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+              int64_t cap, RecRef recRef, const uint32_t* __restrict__ chunkBase,
               uint32_t* __restrict__ perm, uint32_t* permShuffled) {
+  const BmRecord* __restrict__ records = recRef.get();
   permuteRow(g, m, coors, liveCount(numActIn, cap), static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x, records,
              chunkBase, perm, permShuffled);
 }
@@ -1179,9 +1247,10 @@ bmPermutation(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int
 template <bool SUBM>
 __global__ void __launch_bounds__(kRbThreads)
 bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
-        int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+        int64_t pitch, RecRef recRef, const uint32_t* __restrict__ chunkBase,
         const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut,
         uint32_t* __restrict__ staging, RbCount* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
+  const BmRecord* __restrict__ records = recRef.get();
   __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
   const int tap = blockIdx.y;
@@ -1375,7 +1444,8 @@ __device__ __forceinline__ uint32_t nearMembers(const BlockMap& m, const NearBas
 template <int KSEL>
 __global__ void __launch_bounds__(kRbThreads)
 bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
-           BmRecord* records) {
+           RecRef recRef) {
+  BmRecord* records = recRef.get();
   __shared__ unsigned long long masks[kNearGroup][kRbThreads];
   const int n = liveCount(numActIn, cap);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kRbThreads + threadIdx.x;
@@ -1410,10 +1480,11 @@ bmMarkNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_
 template <bool SUBM, int KSEL>
 __global__ void __launch_bounds__(kRbThreads)
 bmProbeNear(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
-            int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+            int64_t pitch, RecRef recRef, const uint32_t* __restrict__ chunkBase,
             uint32_t* __restrict__ perm, uint32_t* permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
             RbCount* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals, int32_t* fillA, int64_t nFillA, int32_t* fillB,
             int64_t nFillB, uint32_t fillBlocks, int32_t* __restrict__ outCoors, uint32_t nRecords) {
+  const BmRecord* __restrict__ records = recRef.get();
   extern __shared__ __attribute__((aligned(16))) unsigned char nearSmem[];
   uint4* group = reinterpret_cast<uint4*>(nearSmem);                                   // [8][kRbThreads] records
   uint32_t* ldsCnt = reinterpret_cast<uint32_t*>(group + kNearGroup * kRbThreads);    // [kVol]
@@ -1516,12 +1587,13 @@ static_assert(1 << kProbeShift == kProbeThreads, "counts per workgroup");
 template <bool SUBM, int K1, int K2, int K3>
 __global__ void __launch_bounds__(kProbeThreads)
 bmProbeFixed(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
-             int64_t pitch, const BmRecord* __restrict__ records, const uint32_t* __restrict__ chunkBase,
+             int64_t pitch, RecRef recRef, const uint32_t* __restrict__ chunkBase,
              uint32_t* __restrict__ perm, uint32_t* permShuffled, int32_t maxNumActOut, uint32_t* __restrict__ staging,
              RbCount* __restrict__ cnt, uint32_t cntPitch, int32_t* fillA, int64_t nFillA, int32_t* fillB,
              int64_t nFillB, uint32_t fillBlocks, uint32_t probeBlocks, int32_t* __restrict__ outCoors,
              uint32_t nRecords, unsigned long long* __restrict__ maskOut, int64_t nMasks, int fixTail,
              int32_t* __restrict__ nbrDirect, int64_t nbrRows, uint32_t* fillState, int handOver) {
+  const BmRecord* __restrict__ records = recRef.get();
   // Besides the staging entries the pass writes what a linked convolution reads: maskOut (SubM, staging rows =
   // rows of the mirrored table) takes the tile masks - a wavefront's 64 inputs are one 64-row tile - and fixTail
   // has the rows between the live count and the capacity set to -1; nbrDirect (strided, index tensor unread)
@@ -1657,6 +1729,12 @@ bmProbeFixed(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int3
 }
 
 size_t alignUp(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
+
+// workgroups of `threads` threads that give every kEmitGroup records a wavefront
+uint32_t emitBlocks(uint32_t nRecords, int threads) {
+  const uint32_t perBlock = static_cast<uint32_t>(threads / 64) * kEmitGroup;
+  return (nRecords + perBlock - 1) / perBlock;
+}
 
 uint32_t nextPow2(uint64_t v) {
   uint64_t p = 1;
@@ -1804,6 +1882,8 @@ bool blockMapFits(const RbGeom& g) {
 
 }  // namespace
 
+size_t mapStateWords(size_t chunkBaseBytes) { return 4 + scanGroups(static_cast<uint32_t>(chunkBaseBytes / 4)) + 1; }
+
 void blockMapBytes(const RbGeom& g, int64_t cap, size_t* records, size_t* chunkBase) {
   *records = *chunkBase = 0;
   const RbWorkspace w = planRulebookWorkspace(g, cap, false, ~static_cast<size_t>(0));
@@ -1938,21 +2018,33 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     const BlockMap m = makeBlockMap(g, &nRecords64);
     // the map lives in the workspace, or in the caller's buffers that carry it from a strided build to the SubM
     // builds on its outputs
-    const bool mapOutside = side.mapRecords && side.mapChunkBase && (!subM || side.useSharedMap);
-    const bool sharedMap = subM && mapOutside;
+    const bool mapOutside = side.mapRecords && side.mapChunkBase;
+    const bool sharedMap = subM && mapOutside && side.useSharedMap;
     auto* records = mapOutside ? static_cast<BmRecord*>(side.mapRecords) : reinterpret_cast<BmRecord*>(ws + w.table);
     auto* perm = reinterpret_cast<uint32_t*>(ws + w.ids);
     auto* chunkBase = mapOutside ? side.mapChunkBase : reinterpret_cast<uint32_t*>(ws + w.ownCnt);
     side.mapWritten = !subM && mapOutside;
-    uint32_t* scanTicket = ownTotals + g.kVol + 1;
     const dim3 perChunk(w.nChunks > 0 ? w.nChunks : 1);
-    uint32_t* permShuffled = ownTotals + g.kVol;
+    const bool near = nearEligible(g, m);
+    const int ksel = near ? fixedKernelShape(g) : 0;
+    // Two maps in turn (no reset pass) when the caller keeps the map and its state between passes and the probe
+    // is the fixed-shape one, which leaves nothing else to zero; a SubM build on a shared map follows the build
+    // that wrote it.
+    const bool twoMaps = mapOutside && side.mapState && side.mapStride > 0 &&
+                         (sharedMap ? side.mapDouble
+                                    : (side.mapStride == static_cast<int64_t>(w.nRecords) && near && ksel != 0 &&
+                                       !side.skipIndex && !side.mapDirty));
+    side.mapDouble = twoMaps;
+    uint32_t* const epochPtr = twoMaps ? side.mapState : nullptr;
+    const uint32_t recStride = twoMaps ? static_cast<uint32_t>(side.mapStride) : 0u;
+    const RecRef recBefore{records, epochPtr, recStride, 0u};  // mark and scan
+    const RecRef recBehind{records, epochPtr, recStride, 1u};  // behind the scan: probe, coordinates, SubM builds on it
+    uint32_t* scanTicket = (twoMaps && !sharedMap) ? side.mapState + 2 : ownTotals + g.kVol + 1;
+    uint32_t* permShuffled = (twoMaps && !sharedMap) ? side.mapState + 1 : ownTotals + g.kVol;
     if (subM && !sharedMap) {
       compactPerm = perm;
       compactPermFlag = permShuffled;
     }
-    const bool near = nearEligible(g, m);
-    const int ksel = near ? fixedKernelShape(g) : 0;
     const size_t nearLds = static_cast<size_t>(kNearGroup) * kRbThreads * sizeof(uint4) + static_cast<size_t>(g.kVol) * 4;
     // A build whose index tensor nobody reads (side.skipIndex) writes table and masks in the probe pass and skips
     // the compaction: for the kernel shapes of the plane probe, a SubM build with the mirrored table staged in
@@ -1970,7 +2062,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     const int64_t clearRecords = sharedMap ? 0 : static_cast<int64_t>(w.nRecords);
     // A build on a shared map with the fixed-shape probe leaves nothing to zero: the probe writes counts and tile
     // masks with plain stores, the compaction sums the counts itself, numIndex is written last.
-    needReset = !(sharedMap && near && ksel != 0 && !directScatter && !resetFill && compactMasks == nullptr);
+    needReset = !((sharedMap || twoMaps) && near && ksel != 0 && !directScatter && !resetFill && compactMasks == nullptr);
     if (needReset)
       hipLaunchKernelGGL(bmReset, fillGrid(clearRecords + (resetFill ? resetFillN / 4 : 0) + 1), block, 0,
                          stream, reinterpret_cast<uint4*>(records), clearRecords,
@@ -1980,38 +2072,39 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
     if (sharedMap) {
       // the strided build that wrote these coordinates marked and scanned this very grid
     } else if (subM) {
-      hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
+      hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, recBefore,
+                         needReset ? nullptr : permShuffled);
     } else if (near) {
       switch (ksel) {
-        case 1: hipLaunchKernelGGL(bmMarkNear<1>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records); break;
-        case 2: hipLaunchKernelGGL(bmMarkNear<2>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records); break;
-        case 3: hipLaunchKernelGGL(bmMarkNear<3>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records); break;
-        case 4: hipLaunchKernelGGL(bmMarkNear<4>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records); break;
-        default: hipLaunchKernelGGL(bmMarkNear<0>, perInput, block, 0, stream, g, m, coors, numActIn, cap, records);
+        case 1: hipLaunchKernelGGL(bmMarkNear<1>, perInput, block, 0, stream, g, m, coors, numActIn, cap, recBefore); break;
+        case 2: hipLaunchKernelGGL(bmMarkNear<2>, perInput, block, 0, stream, g, m, coors, numActIn, cap, recBefore); break;
+        case 3: hipLaunchKernelGGL(bmMarkNear<3>, perInput, block, 0, stream, g, m, coors, numActIn, cap, recBefore); break;
+        case 4: hipLaunchKernelGGL(bmMarkNear<4>, perInput, block, 0, stream, g, m, coors, numActIn, cap, recBefore); break;
+        default: hipLaunchKernelGGL(bmMarkNear<0>, perInput, block, 0, stream, g, m, coors, numActIn, cap, recBefore);
       }
     } else {
-      hipLaunchKernelGGL(bmMarkCandidates, perTap, block, 0, stream, g, m, coors, numActIn, cap, records);
+      hipLaunchKernelGGL(bmMarkCandidates, perTap, block, 0, stream, g, m, coors, numActIn, cap, recBefore);
     }
     // D3D_RULEBOOK_ORDERED_SCAN=1: acquire-release tickets (see bmScan)
     if (sharedMap) {
     } else if (debugEnv("D3D_RULEBOOK_ORDERED_SCAN"))
-      hipLaunchKernelGGL(bmScan<true>, perChunk, block, 0, stream, records, w.nRecords, chunkBase, w.nChunks, scanTicket,
+      hipLaunchKernelGGL(bmScan<true>, perChunk, block, 0, stream, recBefore, w.nRecords, chunkBase, w.nChunks, scanTicket,
                          scanTicket + 1, subM ? nullptr : numActOut, maxNumActOut);
     else
-      hipLaunchKernelGGL(bmScan<false>, perChunk, block, 0, stream, records, w.nRecords, chunkBase, w.nChunks,
+      hipLaunchKernelGGL(bmScan<false>, perChunk, block, 0, stream, recBefore, w.nRecords, chunkBase, w.nChunks,
                          scanTicket, scanTicket + 1, subM ? nullptr : numActOut, maxNumActOut);
     if (!near) {  // the near probe launch carries these passes itself
       if (!subM)
-        hipLaunchKernelGGL(bmEmitCoords, dim3((w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64)), block, 0, stream,
-                           g, m, records, chunkBase, w.nRecords, outCoors, maxNumActOut);
+        hipLaunchKernelGGL(bmEmitCoords, dim3(emitBlocks(w.nRecords, kRbThreads)), block, 0, stream,
+                           g, m, recBehind, chunkBase, w.nRecords, outCoors, maxNumActOut);
       if (subM && !sharedMap)
-        hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, records, chunkBase,
+        hipLaunchKernelGGL(bmPermutation, perInput, block, 0, stream, g, m, coors, numActIn, cap, recBehind, chunkBase,
                            perm, permShuffled);
     }
     if (near) {  // probe workgroups interleaved 1:1 with fill workgroups (index tensor, neighbour table)
       const uint32_t probeBlocks = perInput.x;
       const uint32_t quads = probeBlocks;
-      const uint32_t extra = sharedMap ? 0u : (subM ? probeBlocks : (w.nRecords + kRbThreads / 64 - 1) / (kRbThreads / 64));
+      const uint32_t extra = sharedMap ? 0u : (subM ? probeBlocks : emitBlocks(w.nRecords, kRbThreads));
       const dim3 fused(quads * 2 + extra);
       int32_t* fillB = (nbrOut && nbrRows > 0 && !mirror && !directScatter) ? nbrOut : nullptr;
       int32_t* const probeFillIndex = skipIndex ? nullptr : fillIndex;
@@ -2019,7 +2112,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       nbrFilled = true;
 #define D3D_LAUNCH_PROBE_NEAR(SUBM, KSEL)                                                                          \
   hipLaunchKernelGGL((bmProbeNear<SUBM, KSEL>), fused, block, nearLds, stream, g, m, coors, numActIn, cap, pitch,   \
-                     records, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.cntPitch, nullptr, fillIndex, \
+                     recBehind, chunkBase, perm, permShuffled, maxNumActOut, staging, cnt, w.cntPitch, nullptr, fillIndex, \
                      nIndex, fillB, nFillB, quads, outCoors, w.nRecords)
       // fixed kernel shapes: K1 threads per input; fill workgroups only for what there is to fill
       const int64_t fillItems = (probeFillIndex ? nIndex : 0) + nFillB;
@@ -2027,11 +2120,11 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       if (planeFill > 1024) planeFill = 1024;
       // the fixed-shape probe runs workgroups of kProbeThreads inputs
       const uint32_t fixedBlocks = static_cast<uint32_t>((cap + kProbeThreads - 1) / kProbeThreads > 0 ? (cap + kProbeThreads - 1) / kProbeThreads : 1);
-      const uint32_t fixedExtra = sharedMap ? 0u : (subM ? fixedBlocks : (w.nRecords + kProbeThreads / 64 - 1) / (kProbeThreads / 64));
+      const uint32_t fixedExtra = sharedMap ? 0u : (subM ? fixedBlocks : emitBlocks(w.nRecords, kProbeThreads));
       planeFill = (planeFill * kRbThreads + kProbeThreads - 1) / kProbeThreads;
 #define D3D_LAUNCH_PROBE_PLANE(SUBM, K1, K2, K3)                                                                    \
   hipLaunchKernelGGL((bmProbeFixed<SUBM, K1, K2, K3>), dim3(planeFill + fixedBlocks + fixedExtra), dim3(kProbeThreads), 0, stream, \
-                     g, m, coors, numActIn, cap, pitch, records, chunkBase, perm, permShuffled, maxNumActOut,     \
+                     g, m, coors, numActIn, cap, pitch, recBehind, chunkBase, perm, permShuffled, maxNumActOut,   \
                      (directScatter && skipIndex) ? nullptr : staging, cnt, w.cntPitch, probeFillIndex,             \
                      nIndex, fillB, nFillB, planeFill,                                                               \
                      fixedBlocks, outCoors, w.nRecords, probeMasks ? masks : nullptr, nMasks,                        \
@@ -2058,10 +2151,10 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
 #undef D3D_LAUNCH_PROBE_PLANE
 #undef D3D_LAUNCH_PROBE_NEAR
     } else if (subM) {
-      hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, pitch, records, chunkBase, perm,
+      hipLaunchKernelGGL(bmProbe<true>, perTap, block, 0, stream, g, m, coors, numActIn, cap, pitch, recBehind, chunkBase, perm,
                          permShuffled, maxNumActOut, staging, cnt, w.cntPitch, nullptr);
     } else {
-      hipLaunchKernelGGL(bmProbe<false>, perTap, block, 0, stream, g, m, coors, numActIn, cap, pitch, records, chunkBase, perm,
+      hipLaunchKernelGGL(bmProbe<false>, perTap, block, 0, stream, g, m, coors, numActIn, cap, pitch, recBehind, chunkBase, perm,
                          permShuffled, maxNumActOut, staging, cnt, w.cntPitch, nullptr);
     }
   } else {
