@@ -37,9 +37,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRawBuffer(const void* p, u
 
 // tileMasks: one 64-bit tap mask per 64 output rows, padded with zero entries to a multiple of 8 entries past
 // ceil(outRows / 64) (a workgroup reads the masks of a whole tile at once); null = every tap of every tile.
-// DBG (timing experiments only, results are wrong): 1 no gathers, 2 no MFMA, 4 no row fragment reads,
-// 8 no weight fragment reads, 16 no barrier.
-template <class T, int CIN, int COUT, int MT, int WAVES, int DBG = 0>
+template <class T, int CIN, int COUT, int MT, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES)
 convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
          const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror,
@@ -72,7 +70,6 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
   using Acc = typename Mfma<T>::Acc;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  if constexpr ((DBG & 32) != 0) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -251,9 +248,7 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
         const auto s1 = __builtin_amdgcn_permlane16_swap(a[1], c[1], false, false);
         const u32x4 line = {s0[0], s1[0], s0[1], s1[1]};
         const int64_t row = row0 + m * 16 + r16;
-        if (row < outRows && !(DBG & 128))
-          *reinterpret_cast<u32x4*>(out + static_cast<size_t>(row) * COUT + outCol) = line;
-        if (DBG & 128) asm volatile("" ::"v"(line));
+        if (row < outRows) *reinterpret_cast<u32x4*>(out + static_cast<size_t>(row) * COUT + outCol) = line;
       }
     }
   };
@@ -325,30 +320,25 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
       F(&nxt)[KK] = rowBuf[(m + 1 + PAR) & 1];
       int32_t(&ix)[GPM] = ixBuf[(m + PAR) & 1];
       if (m + 1 < MT) {
-        if constexpr (!(DBG & 4)) readRowGroup(nxt, m + 1, SLOT);
+        readRowGroup(nxt, m + 1, SLOT);
         readIndex(a + 2, m + 1, ixBuf[(m + 1 + PAR) & 1]);
       } else {
         // everything issued before this step has landed: the rows of the next step, this wavefront's part of
         // the weight slice of the step after next, the indices of the step after that
-        waitVmcnt<((DBG & 1) ? 0 : (MT - 1) * GPM) + extraBeforeWait>();
-        if constexpr (!(DBG & 4)) readRowGroup(nxt, 0, SLOT ^ 1);
+        waitVmcnt<(MT - 1) * GPM + extraBeforeWait>();
+        readRowGroup(nxt, 0, SLOT ^ 1);
         readIndex(a + 3, 0, ixBuf[(m + 1 + PAR) & 1]);
       }
 #pragma unroll
       for (int e = m * WREADS; e < (m + 1) * WREADS && e < NQ; ++e)
-        if constexpr (!(DBG & 8)) readWeight(nxtW, e, nextBuf);
+        readWeight(nxtW, e, nextBuf);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
-        if constexpr (!(DBG & 2)) {
-          acc[m][q % NT] = Mfma<T>::k32(curW[q / NT][q % NT], cur[q / NT], acc[m][q % NT]);
-        } else {
-          asm volatile("" ::"v"(curW[q / NT][q % NT]), "v"(cur[q / NT]));
-        }
+        acc[m][q % NT] = Mfma<T>::k32(curW[q / NT][q % NT], cur[q / NT], acc[m][q % NT]);
         __builtin_amdgcn_sched_barrier(0);
         // the fragments of group m have left LDS (the MFMA above waited for them): refill its stage rows
-        if (q < GPM && !(DBG & 1)) gatherOne(m * GPM + q, ix[q], partOff, SLOT);
-        if (q < GPM && (DBG & 1)) asm volatile("" ::"v"(ix[q]));
+        if (q < GPM) gatherOne(m * GPM + q, ix[q], partOff, SLOT);
         if (q >= GPM) {
           const int u = m * FREE + q - GPM;         // ordinal of this free slot within the step
           if (u == 0) loadIndex(a + 4);
@@ -359,14 +349,10 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
     }
     wbuf = nextBuf;
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_s_barrier();
     return lastOfTile;
   };
 
-  if constexpr ((DBG & 64) != 0) {
-    for (int pos = 0; pos < nMine; ++pos) storeTile(pos);
-    return;
-  }
   for (int a = 0;; a += 2) {
     if (step(a, std::integral_constant<int, 0>{}, wtsA, wtsB)) {
       storeTile(walkMul.pos);
@@ -380,7 +366,7 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
   waitVmcnt<0>();                                   // loads issued for steps that do not exist, and the stores
 }
 
-template <class T, int CIN, int COUT, int MT, int WAVES, int DBG = 0>
+template <class T, int CIN, int COUT, int MT, int WAVES>
 int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
   constexpr int CS = CIN > 64 ? 64 : CIN;
   constexpr int WM = 16 * MT, TM = WM * WAVES;
@@ -394,7 +380,7 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
       static_cast<uint64_t>(a.outRows) + TM >= 0x3FFFFFFFull)
     return D3D_ERR_UNSUPPORTED;                         // 32-bit buffer offsets
   static std::atomic<size_t> granted{64 * 1024};
-  const int32_t rc = grantLds(&convPipe<T, CIN, COUT, MT, WAVES, DBG>, lds, &granted);
+  const int32_t rc = grantLds(&convPipe<T, CIN, COUT, MT, WAVES>, lds, &granted);
   if (rc != D3D_OK) return rc;
   const int tiles = static_cast<int>((a.outRows + TM - 1) / TM);
   // persistent workgroups: as many as the CUs can hold at this LDS footprint, never more than there are tiles
@@ -403,7 +389,7 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
   if (perCu < 1) perCu = 1;
   int blocks = (tiles + 7) / 8 * 8;
   if (blocks > 256 * perCu) blocks = 256 * perCu;
-  hipLaunchKernelGGL((convPipe<T, CIN, COUT, MT, WAVES, DBG>), dim3(static_cast<unsigned>(blocks)), dim3(64 * WAVES),
+  hipLaunchKernelGGL((convPipe<T, CIN, COUT, MT, WAVES>), dim3(static_cast<unsigned>(blocks)), dim3(64 * WAVES),
                      lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
                      static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, pitch, a.tapMirror, a.tileMasks, a.kVol,
                      a.inRows, a.outRows, a.relu, tiles);
@@ -417,7 +403,11 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
 // tile halves.  32 -> 32 takes 8 wavefronts as well (two workgroups of 78 KB per CU, 16 wavefronts): 38 us against
 // 41 with 4, 40 with three 4-wavefront workgroups per CU, 41 with 128-row and 42 with 48-row wavefront tiles; with gathers and MFMAs
 // both taken out of it the kernel still runs 27 us on that layer (25 with the table reads served from cache), so
-// what is left is the per-step bookkeeping of a 32-channel step, not a memory or matrix limit.  Layers with few
+// what is left is the per-step bookkeeping of a 32-channel step, not a memory or matrix limit.  Two taps per step
+// (a stage row holding the neighbours under two taps side by side, the step of a 64-channel layer) measured slower
+// on both 32-channel layers in every tile shape tried (32 -> 32: 44-58 us against 37.5; 32 -> 64: 45-57 against
+// 36): the stage doubles, one workgroup fits a CU instead of two, and the layer needs the wavefronts more than
+// the longer steps.  Layers with few
 // rows (the 128-channel stages: 47 000 rows are 186 tiles of 256 rows for 256 CUs) pick the workgroup shape by
 // tile count: the time of a layer that fits one round is that of ONE tile, so 248 tiles of 192 rows beat 186 of
 // 256 (48 us against 55), and there four wavefronts of 48 rows - one per SIMD, three 16-row groups each - beat
