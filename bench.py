@@ -370,6 +370,76 @@ def main():
                              "lanes of their own, events straight between the lanes",
                      "outputs_equal_full_pass": bool(torch.equal(y3.feats, y.feats))}
             del net3
+        # further figures beside `value` (same kernels, other conditions): what a caller gets who binds the operators
+        # unchanged (`reference_contract`), replays that alternate between two different clouds, and capacities
+        # with head-room over the live counts
+        def replay_ms(graphs, steps):
+            for g in graphs:
+                g.replay()
+            stream.synchronize()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(steps):
+                graphs[i % len(graphs)].replay()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3 / steps
+
+        def captured(network, inp):
+            for _ in range(2):
+                out_t = network.forward(inp)
+            stream.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                out_t = network.forward(inp)
+            return g, out_t
+
+        extra = {}
+        if not args.no_graph and not args.no_fused:
+            # (a) no d3d_link_*, no D3D_OPT_PERSISTENT_INDEX: every rulebook operator fills its whole index tensor
+            # with -1 (reference: trt/spconv/index.cu:352-354), every convolution derives its table from the tensor
+            net_r = layers.SparseBackbone(specs, weights, caps, dtype=dtype, overlap=not args.no_overlap,
+                                          extensions=False)
+            g_r, y_r = captured(net_r, x)
+            ms_r = replay_ms([g_r], args.steps)
+            extra["reference_contract"] = {
+                "ms_per_step": round(ms_r, 4), "effective_tflops": round(total_flops / (ms_r * 1e-3) / 1e12, 2),
+                "what": "the same pass with the operators as the reference's contract alone describes them: no "
+                        "d3d_link_rulebook / d3d_link_coords, no D3D_OPT_PERSISTENT_INDEX - index tensors filled with "
+                        "-1 at capacity on every enqueue, neighbour tables derived from the index tensor per enqueue",
+                "outputs_equal_full_pass": bool(torch.equal(y_r.feats, y.feats))}
+            del net_r, g_r
+            # (b) two clouds in turn: the full cloud and one with ~8 % fewer voxels (the first rows of a shuffled
+            # copy), each in buffers of its own at the same capacities; replays alternate, so the incremental fill of
+            # the persistent index tensors and the tile masks see change between passes
+            n_b = int(n * 0.92)
+            pick = np.sort(np.random.default_rng(5).permutation(n)[:n_b])
+            x_b = layers.make_input(cfg["coords"][pick], feats[pick], cfg["grid"], dtype=dtype, capacity=n)
+            g_b, y_b = captured(net, x_b)
+            g_a, y_a = captured(net, x)
+            ms_ab = replay_ms([g_a, g_b], 2 * (args.steps // 2 + 1))
+            g_a.replay()
+            stream.synchronize()
+            extra["alternating_clouds"] = {
+                "ms_per_step": round(ms_ab, 4), "voxels": [n, n_b],
+                "what": "graph replays alternating between two clouds (the second a random 92 % subset of the "
+                        "first) through the same operators and capacities",
+                "full_cloud_output_unchanged": bool(torch.equal(y_a.feats, ref_out))}
+            del g_b, x_b
+            # (c) capacities at 1.5 x the live counts (input rows and every strided layer's maxNumActOut)
+            counts15 = {k: int(v * 1.5) for k, v in counts.items()}
+            caps15 = layers.plan_capacities(specs, int(n * 1.5), counts15)
+            net_c = layers.SparseBackbone(specs, weights, caps15, dtype=dtype, overlap=not args.no_overlap)
+            x_c = layers.make_input(cfg["coords"], feats, cfg["grid"], dtype=dtype, capacity=int(n * 1.5))
+            g_c, y_c = captured(net_c, x_c)
+            ms_c = replay_ms([g_c], args.steps)
+            n_c = int(y_c.num_act.item())
+            extra["capacity_1p5x"] = {
+                "ms_per_step": round(ms_c, 4), "capacities": caps15,
+                "what": "the same cloud with every row capacity at 1.5 x the live count (kernels are launched at "
+                        "capacity)",
+                "outputs_equal_full_pass": bool(n_c == int(y.num_act.item()) and
+                                                torch.equal(y_c.feats[:n_c], y.feats[:n_c]))}
+            del net_c, g_c, x_c
         n_final = int(y.num_act.item())
         gpu_coords = y.coors[:n_final].cpu().numpy()
         gpu_feats = y.feats[:n_final].float().cpu().numpy() if dtype != torch.int8 else y.feats[:n_final].cpu().numpy()
@@ -458,6 +528,9 @@ def main():
         "rulebook_ms": {k: round(t, 4) for k, t in rulebook_ms.items()},
         "index_unused": fused,
         "native_schedule": sched,
+        "reference_contract": extra.get("reference_contract"),
+        "alternating_clouds": extra.get("alternating_clouds"),
+        "capacity_1p5x": extra.get("capacity_1p5x"),
         "roofline": roofline,
         "rooflines": rooflines,
         "measured_peak": peaks,

@@ -135,9 +135,9 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
 
 // Out-major neighbour table of one rulebook: nbr[tap, row] = gathered input row
 // or -1, rows = maxNumActOut.  Built from the index tensor (optionally with the
-// gather and scatter rows swapped for an inverse convolution).
+// gather and scatter rows swapped for an inverse convolution); pairs whose gather row lies outside [0, inRows) are dropped.
 int32_t launchBuildNeighbours(const int32_t* index, int64_t rowLen, const int32_t* numIndex, bool inverse, int kVol,
-                              int64_t outRows, int32_t* nbr, hipStream_t stream);
+                              int64_t outRows, int64_t inRows, int32_t* nbr, hipStream_t stream);
 
 struct ConvArgs {
   int32_t dtype;          // D3D_FLOAT / D3D_HALF / D3D_BF16 / D3D_INT8

@@ -41,7 +41,8 @@ __global__ void __launch_bounds__(256) nbrFill(int32_t* nbr, int64_t n) {
 
 __global__ void __launch_bounds__(256)
 nbrScatter(const int32_t* __restrict__ gather, const int32_t* __restrict__ scatter, const int32_t* __restrict__ tapRow,
-           const int32_t* __restrict__ numIndex, int64_t rowLen, int kVol, int64_t outRows, int32_t* __restrict__ nbr) {
+           const int32_t* __restrict__ numIndex, int64_t rowLen, int kVol, int64_t outRows, int64_t inRows,
+           int32_t* __restrict__ nbr) {
   int64_t n = *numIndex;
   if (n > rowLen) n = rowLen;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
@@ -50,9 +51,13 @@ nbrScatter(const int32_t* __restrict__ gather, const int32_t* __restrict__ scatt
     if (t < 0 || t >= kVol) continue;  // padding slot
     const int32_t o = scatter[j];
     if (o < 0 || o >= outRows) continue;
+    // a gather row outside the input is no neighbour: the table holds -1 or rows that exist, nothing else (the
+    // kernels that turn an entry into a buffer offset rely on that)
+    const int32_t i = gather[j];
+    if (i < 0 || i >= inRows) continue;
     // An index tensor that names two inputs for one (tap, output) - duplicate coordinates, a tensor of other
     // origin - keeps the higher input row: one neighbour per (tap, output), the same one on every run.
-    atomicMax(&nbr[static_cast<int64_t>(t) * outRows + o], gather[j]);
+    atomicMax(&nbr[static_cast<int64_t>(t) * outRows + o], i);
   }
 }
 
@@ -318,7 +323,7 @@ int32_t launchPadRows(const void* in, int64_t rows, int inBytes, int outBytes, v
 }
 
 int32_t launchBuildNeighbours(const int32_t* index, int64_t rowLen, const int32_t* numIndex, bool inverse, int kVol,
-                              int64_t outRows, int32_t* nbr, hipStream_t stream) {
+                              int64_t outRows, int64_t inRows, int32_t* nbr, hipStream_t stream) {
   const int64_t n = static_cast<int64_t>(kVol) * outRows;
   if (n <= 0) return D3D_OK;
   int fillBlocks = static_cast<int>((n + 255) / 256);
@@ -330,7 +335,7 @@ int32_t launchBuildNeighbours(const int32_t* index, int64_t rowLen, const int32_
   if (blocks > 4096) blocks = 4096;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(nbrScatter, dim3(blocks), dim3(256), 0, stream, gather, scatter, index + 2 * rowLen, numIndex,
-                     rowLen, kVol, outRows, nbr);
+                     rowLen, kVol, outRows, inRows, nbr);
   D3D_HIP_CHECK(hipGetLastError());
   return D3D_OK;
 }

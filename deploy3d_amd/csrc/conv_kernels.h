@@ -105,7 +105,7 @@ template <class T, int CIN, int COUT, int MT, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES)
 convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
          const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror, const T* __restrict__ zeros, int kVol,
-         int64_t inRows, int64_t outRows, int relu, int tileBlocks) {
+         int64_t inRows, int64_t outRows, int relu, int tileBlocks, int xcdShift) {
   constexpr int THREADS = 64 * WAVES;
   constexpr int WM = 16 * MT;            // rows per wavefront
   constexpr int TM = WAVES * WM;         // rows per workgroup
@@ -126,10 +126,11 @@ convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kgrp = lane >> 4;
-  // Workgroups are dealt to the 8 XCDs round-robin; handing XCD x the x-th contiguous eighth of the tiles
+  // Workgroups are dealt to the XCDs round-robin; handing XCD x the x-th contiguous part of the tiles
   // keeps neighbouring tiles, which gather many of the same rows, behind the same L2.
-  const int perXcd = (tileBlocks + 7) / 8;
-  const int tile = (blockIdx.x & 7) * perXcd + (blockIdx.x >> 3);
+  const int nXcd = 1 << xcdShift;
+  const int perXcd = (tileBlocks + nXcd - 1) >> xcdShift;
+  const int tile = (blockIdx.x & (nXcd - 1)) * perXcd + (blockIdx.x >> xcdShift);
   if (tile >= tileBlocks) return;        // workgroup-uniform, before any barrier
   const int64_t row0 = static_cast<int64_t>(tile) * TM;
   const int32_t* nb = nbT + wave * WM;   // this wavefront's columns of the [kVol][TM] neighbour tile
@@ -284,7 +285,8 @@ template <class T, int CIN, int COUT, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES)
 convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf,
                  const float* __restrict__ bias, const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror,
-                 const T* __restrict__ zeros, int kVol, int64_t inRows, int64_t outRows, int relu, int groups) {
+                 const T* __restrict__ zeros, int kVol, int64_t inRows, int64_t outRows, int relu, int groups,
+                 int xcdShift) {
   constexpr int THREADS = 64 * WAVES;
   constexpr int MT = 1;
   constexpr int NT = COUT / 16;
@@ -317,12 +319,13 @@ convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restr
     for (int kk = 0; kk < KK; ++kk) dst[0][kk] = *reinterpret_cast<const F*>(rowPtr + kk * KSTEP);
   };
 
-  // Workgroups are dealt to the 8 XCDs round-robin; XCD x takes the x-th contiguous eighth of the row groups,
+  // Workgroups are dealt to the XCDs round-robin; XCD x takes the x-th contiguous part of the row groups,
   // so neighbouring groups, which gather many of the same rows, meet behind the same L2.
-  const int wavesPerXcd = (gridDim.x / 8) * WAVES;
-  const int perXcd = (groups + 7) / 8;
-  const int xcd = blockIdx.x & 7;
-  for (int local = (blockIdx.x >> 3) * WAVES + wave; local < perXcd; local += wavesPerXcd) {
+  const int nXcd = 1 << xcdShift;
+  const int wavesPerXcd = (gridDim.x >> xcdShift) * WAVES;
+  const int perXcd = (groups + nXcd - 1) >> xcdShift;
+  const int xcd = blockIdx.x & (nXcd - 1);
+  for (int local = (blockIdx.x >> xcdShift) * WAVES + wave; local < perXcd; local += wavesPerXcd) {
     const int group = xcd * perXcd + local;
     if (group >= groups) break;
     const int64_t row0 = static_cast<int64_t>(group) * 16;
@@ -459,7 +462,7 @@ __global__ void __launch_bounds__(64 * WAVES)
 convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
            const float* __restrict__ requantM, const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror,
            const unsigned long long* __restrict__ tileMasks, const T* __restrict__ zeros, int kVol, int64_t inRows,
-           int64_t outRows, int relu, int tileBlocks) {
+           int64_t outRows, int relu, int tileBlocks, int xcdShift) {
   constexpr int THREADS = 64 * WAVES;
   constexpr int ES = static_cast<int>(sizeof(T));              // 2: fp16 / bf16, 1: int8
   constexpr int CS = CIN / KS;                                 // input channels per step (a tap takes KS steps)
@@ -514,9 +517,10 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
   const uint32_t rowLimit = static_cast<uint32_t>(inRows);   // the launcher keeps inRows * row bytes below 4 GiB
   const uintptr_t zeroBase = reinterpret_cast<uintptr_t>(zeros);
 
-  const int perXcd = (tileBlocks + 7) / 8;
-  const int xcd = blockIdx.x & 7;
-  for (int local = blockIdx.x >> 3; local < perXcd; local += gridDim.x >> 3) {
+  const int nXcd = 1 << xcdShift;
+  const int perXcd = (tileBlocks + nXcd - 1) >> xcdShift;
+  const int xcd = blockIdx.x & (nXcd - 1);
+  for (int local = blockIdx.x >> xcdShift; local < perXcd; local += gridDim.x >> xcdShift) {
     const int tile = xcd * perXcd + local;
     if (tile >= tileBlocks) break;                     // workgroup-uniform
     const int64_t row0 = static_cast<int64_t>(tile) * TM + wave * WM;
@@ -825,6 +829,26 @@ convStaged(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ 
 
 constexpr size_t kLdsLimit = 160 * 1024;
 
+// Compute units of the device the process runs on and log2 of the number of XCDs they are spread over, read once
+// from the runtime.  Workgroups are dealt to the XCDs of a partition round-robin, and the tile orders of the
+// kernels above follow that: a gfx950 XCD has 32 active compute units, so a whole MI355X reports 256 = 8 XCDs and
+// its partition modes 128 / 64 / 32 = 4 / 2 / 1.
+struct ChipLayout {
+  int cus;
+  int xcdShift;
+};
+inline ChipLayout chipLayout() {
+  static const ChipLayout layout = [] {
+    int dev = 0, cus = 256;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+      cus = prop.multiProcessorCount;
+    const int xcds = cus / 32;
+    return ChipLayout{cus, xcds >= 8 ? 3 : (xcds >= 4 ? 2 : (xcds >= 2 ? 1 : 0))};
+  }();
+  return layout;
+}
+
 template <int CIN, int COUT>
 constexpr size_t mfmaLds(int kVol, int rows, size_t elem) {
   return static_cast<size_t>(2) * CIN * COUT * elem + static_cast<size_t>(kVol) * rows * 4 +
@@ -855,11 +879,14 @@ int32_t launchMfmaTile(const ConvArgs& a, hipStream_t stream) {
   const int32_t rc = grantLds(&convMfma<T, CIN, COUT, MT, WAVES>, lds, &granted);
   if (rc != D3D_OK) return rc;
   const int tiles = static_cast<int>((a.outRows + TM - 1) / TM);
-  const int perXcd = (tiles + 7) / 8;
-  hipLaunchKernelGGL((convMfma<T, CIN, COUT, MT, WAVES>), dim3(static_cast<unsigned>(perXcd * 8)), dim3(64 * WAVES),
+  const ChipLayout chip = chipLayout();
+  const int nXcd = 1 << chip.xcdShift;
+  const int perXcd = (tiles + nXcd - 1) / nXcd;
+  hipLaunchKernelGGL((convMfma<T, CIN, COUT, MT, WAVES>), dim3(static_cast<unsigned>(perXcd * nXcd)), dim3(64 * WAVES),
                      lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
                      static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, a.nbrPitch > 0 ? a.nbrPitch : a.outRows,
-                     a.tapMirror, static_cast<const T*>(a.zeros), a.kVol, a.inRows, a.outRows, a.relu, tiles);
+                     a.tapMirror, static_cast<const T*>(a.zeros), a.kVol, a.inRows, a.outRows, a.relu, tiles,
+                     chip.xcdShift);
   return D3D_OK;
 }
 
@@ -871,18 +898,21 @@ int32_t launchMfmaResident(const ConvArgs& a, hipStream_t stream) {
   const int32_t rc = grantLds(&convMfmaResident<T, CIN, COUT, WAVES>, lds, &granted);
   if (rc != D3D_OK) return rc;
   const int groups = static_cast<int>((a.outRows + 15) / 16);
-  // persistent workgroups: as many as fit on the 256 CUs at this LDS footprint, but no more than there is work
+  // persistent workgroups: as many as fit on the CUs at this LDS footprint, but no more than there is work
+  const ChipLayout chip = chipLayout();
+  const int nXcd = 1 << chip.xcdShift;
   int perCu = static_cast<int>(kLdsLimit / (lds + 1024));
   if (perCu < 1) perCu = 1;
   if (perCu > 2) perCu = 2;  // 16 wavefronts each
-  int blocks = 256 * perCu;
+  int blocks = chip.cus / nXcd * nXcd * perCu;
   const int needed = (groups + WAVES - 1) / WAVES;
-  if (blocks > needed) blocks = (needed + 7) / 8 * 8;
-  if (blocks < 8) blocks = 8;
+  if (blocks > needed) blocks = (needed + nXcd - 1) / nXcd * nXcd;
+  if (blocks < nXcd) blocks = nXcd;
   hipLaunchKernelGGL((convMfmaResident<T, CIN, COUT, WAVES>), dim3(static_cast<unsigned>(blocks)), dim3(64 * WAVES),
                      lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
                      static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, a.nbrPitch > 0 ? a.nbrPitch : a.outRows,
-                     a.tapMirror, static_cast<const T*>(a.zeros), a.kVol, a.inRows, a.outRows, a.relu, groups);
+                     a.tapMirror, static_cast<const T*>(a.zeros), a.kVol, a.inRows, a.outRows, a.relu, groups,
+                     chip.xcdShift);
   return D3D_OK;
 }
 
@@ -899,17 +929,19 @@ int32_t launchStagedCfg(const ConvArgs& a, hipStream_t stream) {
   const int32_t rc = grantLds(&convStaged<T, CIN, COUT, KS, MT, WAVES, NS, RESIDENT>, lds, &granted);
   if (rc != D3D_OK) return rc;
   const int tiles = static_cast<int>((a.outRows + TM - 1) / TM);
-  int blocks = (tiles + 7) / 8 * 8;
+  const ChipLayout chip = chipLayout();
+  const int nXcd = 1 << chip.xcdShift;
+  int blocks = (tiles + nXcd - 1) / nXcd * nXcd;
   if (RESIDENT) {  // persistent workgroups share one weight load
     int perCu = static_cast<int>(kLdsLimit / lds);
     if (perCu > 2) perCu = 2;
-    if (blocks > 256 * perCu) blocks = 256 * perCu;
+    if (blocks > chip.cus / nXcd * nXcd * perCu) blocks = chip.cus / nXcd * nXcd * perCu;
   }
   hipLaunchKernelGGL((convStaged<T, CIN, COUT, KS, MT, WAVES, NS, RESIDENT>), dim3(static_cast<unsigned>(blocks)),
                      dim3(64 * WAVES), lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
                      static_cast<const T*>(a.weightsMfma), a.bias, a.requantM, a.nbr,
                      a.nbrPitch > 0 ? a.nbrPitch : a.outRows, a.tapMirror, a.tileMasks, static_cast<const T*>(a.zeros),
-                     a.kVol, a.inRows, a.outRows, a.relu, tiles);
+                     a.kVol, a.inRows, a.outRows, a.relu, tiles, chip.xcdShift);
   return D3D_OK;
 }
 

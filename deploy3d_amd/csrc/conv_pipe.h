@@ -42,7 +42,7 @@ __global__ void __launch_bounds__(64 * WAVES)
 convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
          const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror,
          const unsigned long long* __restrict__ tileMasks, int kVol, int64_t inRows, int64_t outRows, int relu,
-         int tileBlocks) {
+         int tileBlocks, int xcdShift) {
   constexpr int THREADS = 64 * WAVES;
   constexpr int ES = static_cast<int>(sizeof(T));
   constexpr int CS = CIN > 64 ? 64 : CIN;                      // input channels per step; a tap takes KS steps
@@ -96,11 +96,12 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
     idxRow[i] = static_cast<uint32_t>(wave * WM + (p % GL) * RPI + p / GL);
   }
 
-  // ---- this workgroup's tiles: XCD x serves the x-th contiguous eighth of the tiles (neighbouring tiles gather
+  // ---- this workgroup's tiles: XCD x serves the x-th contiguous part of the tiles (neighbouring tiles gather
   // many of the same rows: they should meet behind one L2); inside it, workgroups take tiles round robin ----
-  const int perXcd = (tileBlocks + 7) / 8;
-  const int xcd = blockIdx.x & 7;
-  const int firstLocal = blockIdx.x >> 3, strideLocal = gridDim.x >> 3;
+  const int nXcd = 1 << xcdShift;
+  const int perXcd = (tileBlocks + nXcd - 1) >> xcdShift;
+  const int xcd = blockIdx.x & (nXcd - 1);
+  const int firstLocal = blockIdx.x >> xcdShift, strideLocal = gridDim.x >> xcdShift;
   int nMine = 0;
   if (firstLocal < perXcd) {
     int lastLocal = perXcd - 1;
@@ -387,12 +388,14 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
   int perCu = static_cast<int>(kLdsLimit / lds);
   if (perCu > 2) perCu = 2;
   if (perCu < 1) perCu = 1;
-  int blocks = (tiles + 7) / 8 * 8;
-  if (blocks > 256 * perCu) blocks = 256 * perCu;
+  const ChipLayout chip = chipLayout();
+  const int nXcd = 1 << chip.xcdShift;
+  int blocks = (tiles + nXcd - 1) / nXcd * nXcd;
+  if (blocks > chip.cus / nXcd * nXcd * perCu) blocks = chip.cus / nXcd * nXcd * perCu;
   hipLaunchKernelGGL((convPipe<T, CIN, COUT, MT, WAVES>), dim3(static_cast<unsigned>(blocks)), dim3(64 * WAVES),
                      lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
                      static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, pitch, a.tapMirror, a.tileMasks, a.kVol,
-                     a.inRows, a.outRows, a.relu, tiles);
+                     a.inRows, a.outRows, a.relu, tiles, chip.xcdShift);
   return D3D_OK;
 }
 
@@ -427,13 +430,14 @@ int32_t launchPipeShape(const ConvArgs& a, hipStream_t stream) {
     int64_t bestCost = 0;
     for (int c = 0; c < 3; ++c) {
       const int64_t tm = kCand[c][0] * kCand[c][1], tiles = (a.outRows + tm - 1) / tm;
-      const int64_t cost = (tiles + 255) / 256 * tm;  // rows the busiest CU multiplies
+      const int64_t cus = chipLayout().cus;
+      const int64_t cost = (tiles + cus - 1) / cus * tm;  // rows the busiest CU multiplies
       if (c == 0 || cost < bestCost) {
         best = c;
         bestCost = cost;
       }
     }
-    if (best == 1 && (a.outRows + 191) / 192 <= 256) best = 3;
+    if (best == 1 && (a.outRows + 191) / 192 <= chipLayout().cus) best = 3;
     if (const char* force = debugEnv("D3D_CONV_PIPE_SHAPE")) {  // "rows,wavefronts" of one candidate (tests)
       for (int c = 0; c < 4; ++c)
         if (std::atoi(force) == kCand[c][0] && std::strchr(force, ',') &&

@@ -4,6 +4,8 @@
 //
 // Reference life cycle being mirrored: SPConvIdxPlugin (trt/spconv/index_trt.cu:52-249)
 // and SPConvMMPlugin (trt/spconv/mm_trt.cu:39-206).
+#include <dlfcn.h>
+
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -178,6 +180,7 @@ struct RulebookLink {
   int kVol = 0;
   int64_t outRows = 0, rowLen = 0;
   bool tableValid = false, masksValid = false;
+  bool indexWritten = true;       // false: the last enqueue left the index tensor unwritten (D3D_OPT_INDEX_UNUSED)
   // incremental fill: index tensor that holds a complete earlier pass of this operator
   const void* primedIndex = nullptr;
   int64_t primedRowLen = 0;
@@ -200,6 +203,45 @@ struct RulebookLink {
 };
 
 size_t maskEntries(int64_t outRows) { return static_cast<size_t>((outRows + 63) / 64 + 8); }
+
+// Profiler ranges around an operator's enqueue (reference analogue: the per-layer profiler of
+// deploy3d/symfun/trt_utils/trt_module.py:20-44).  Off unless D3D_ROCTX is set in a process that enabled the
+// debug switches; the tracing library is looked up at run time, so the engine does not link against it.
+struct RoctxRange {
+  typedef int (*PushFn)(const char*);
+  typedef int (*PopFn)();
+  static void lookup(PushFn* push, PopFn* pop) {
+    static PushFn pushFn = nullptr;
+    static PopFn popFn = nullptr;
+    static const bool tried = [] {
+      if (!debugEnv("D3D_ROCTX")) return true;
+      void* lib = dlopen("libroctx64.so", RTLD_NOW | RTLD_GLOBAL);
+      if (!lib) lib = dlopen("librocprofiler-sdk-roctx.so", RTLD_NOW | RTLD_GLOBAL);
+      if (lib) {
+        pushFn = reinterpret_cast<PushFn>(dlsym(lib, "roctxRangePushA"));
+        popFn = reinterpret_cast<PopFn>(dlsym(lib, "roctxRangePop"));
+      }
+      return true;
+    }();
+    (void)tried;
+    *push = pushFn;
+    *pop = popFn;
+  }
+  PopFn pop = nullptr;
+  explicit RoctxRange(const char* name) {
+    PushFn push = nullptr;
+    lookup(&push, &pop);
+    if (push && pop) push(name); else pop = nullptr;
+  }
+  ~RoctxRange() {
+    if (pop) pop();
+  }
+};
+
+bool streamIsCapturing(hipStream_t stream) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+}
 
 // ---------------------------------------------------------------------------
 // packed little-endian blob reader
@@ -336,8 +378,8 @@ struct IdxPlugin final : d3d_plugin {
     }
     if (option != D3D_OPT_PERSISTENT_INDEX) return d3d_plugin::setOption(option, value);
     std::lock_guard<std::mutex> lock(link->mutex);
-    if (value) {
-      int32_t rc = link->fillState.reserve(256);
+    if (value && !link->fillState.ptr) {
+      int32_t rc = link->fillState.reallocZeroed(256);
       if (rc != D3D_OK) return rc;
     }
     persistentIndex = value != 0;
@@ -468,6 +510,7 @@ struct IdxPlugin final : d3d_plugin {
     inGrid[0] = inDesc[2].dims[0];
     for (int i = 0; i < nd; ++i) inGrid[1 + i] = inDesc[2].dims[2 + i];
     const RbGeom g = geometry(grid, inGrid);
+    const RoctxRange range(subM ? "d3d rulebook (submanifold)" : "d3d rulebook (strided)");
     std::lock_guard<std::mutex> lock(link->mutex);
     RbSide side{};
     const size_t tableBytes = static_cast<size_t>(kVol()) * static_cast<size_t>(maxNumActOut) * sizeof(int32_t);
@@ -536,6 +579,11 @@ struct IdxPlugin final : d3d_plugin {
       }
     }
     link->tableValid = link->masksValid = false;
+    // An enqueue on a stream that is being captured runs later, if ever: it must not make the tensor count as
+    // holding a complete pass unless an executed enqueue had already made it so.
+    hipStreamCaptureStatus captureNow = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(stream, &captureNow);
+    const bool wasPrimed = side.incrementalFill;
     link->primedIndex = nullptr;
     int32_t rc = launchRulebook(g, subM, static_cast<const int32_t*>(inputs[0]),
                                 static_cast<const int32_t*>(inputs[1]), cap, maxNumActOut,
@@ -550,8 +598,9 @@ struct IdxPlugin final : d3d_plugin {
       link->outRows = maxNumActOut;
       link->rowLen = rowLen;
       link->tableValid = withTable;
+      link->indexWritten = side.indexWritten;
       link->masksValid = withTable && side.masksWritten;
-      if (side.fillState && side.indexWritten) {
+      if (side.fillState && side.indexWritten && (captureNow == hipStreamCaptureStatusNone || wasPrimed)) {
         link->primedIndex = outputs[0];
         link->primedRowLen = rowLen;
       }
@@ -884,6 +933,7 @@ struct MMPlugin final : d3d_plugin {
       int32_t rc = configure(inDesc, 1, nullptr, 0);
       if (rc != D3D_OK) return rc;
     }
+    const RoctxRange range("d3d convolution");
     const int64_t rowLen = inDesc[3].dims[1];  // numIndicesMax, mm_trt.cu:169
     const int64_t outRows = outDesc[0].dims[0];
     const int32_t* nbr = nullptr;
@@ -898,13 +948,28 @@ struct MMPlugin final : d3d_plugin {
       }
     }
     int32_t rc = D3D_OK;
+    if (!nbr && held) {
+      // the table cannot be used (other shapes, an inverse convolution): the index tensor is all there is to go
+      // by - unless the operator it is linked to left exactly that tensor unwritten on its last enqueue
+      std::lock_guard<std::mutex> lock(held->mutex);
+      if (!held->indexWritten && held->index == inputs[3]) {
+        setError("SPConvMM: the linked rulebook operator left this index tensor unwritten (D3D_OPT_INDEX_UNUSED) "
+                 "and its table does not fit this convolution");
+        return D3D_ERR_UNSUPPORTED;
+      }
+    }
     if (!nbr) {  // the index tensor is all there is to go by: derive the table from it
       if (!derived) derived = std::make_shared<DeviceBuffer>();
       const size_t bytes = static_cast<size_t>(kernelVol) * static_cast<size_t>(outRows > 0 ? outRows : 1) * sizeof(int32_t);
+      if (derived->bytes < bytes && streamIsCapturing(stream)) {
+        setError("SPConvMM: the table derived from the index tensor needs %zu bytes that were not reserved before the "
+                 "capture (configure the node at these shapes, or enqueue it once, first)", bytes);
+        return D3D_ERR_UNSUPPORTED;
+      }
       rc = derived->reserve(bytes);
       if (rc != D3D_OK) return rc;
       rc = launchBuildNeighbours(static_cast<const int32_t*>(inputs[3]), rowLen, static_cast<const int32_t*>(inputs[4]),
-                                 inverse, kernelVol, outRows, static_cast<int32_t*>(derived->ptr), stream);
+                                 inverse, kernelVol, outRows, inDesc[0].dims[0], static_cast<int32_t*>(derived->ptr), stream);
       if (rc != D3D_OK) return rc;
       nbr = static_cast<const int32_t*>(derived->ptr);
     }
@@ -923,7 +988,12 @@ struct MMPlugin final : d3d_plugin {
                                                      debugEnv("D3D_CONV_NO_PAD") == nullptr))) {  // narrow layer: widen the rows, then MFMA
       if (!widened) widened = std::make_shared<DeviceBuffer>();
       const int es = dtypeBytes(dtype);
-      rc = widened->reserve(static_cast<size_t>(a.inRows > 0 ? a.inRows : 1) * dev->cinMfma * es);
+      const size_t wideBytes = static_cast<size_t>(a.inRows > 0 ? a.inRows : 1) * dev->cinMfma * es;
+      if (widened->bytes < wideBytes && streamIsCapturing(stream)) {
+        setError("SPConvMM: %zu bytes for the widened input rows were not reserved before the capture", wideBytes);
+        return D3D_ERR_UNSUPPORTED;
+      }
+      rc = widened->reserve(wideBytes);
       if (rc != D3D_OK) return rc;
       rc = launchPadRows(inputs[0], a.inRows, cin * es, dev->cinMfma * es, widened->ptr, stream);
       if (rc != D3D_OK) return rc;
@@ -1343,6 +1413,14 @@ int32_t d3d_link_rulebook(d3d_plugin* mm, d3d_plugin* idx) {
   }
   if (r->kVol() != m->kernelVol) {
     setError("d3d_link_rulebook: kernel volume %d of the convolution, %d of the rulebook", m->kernelVol, r->kVol());
+    return D3D_ERR_BAD_ARG;
+  }
+  // The table the rulebook operator writes has maxNumActOut rows of ITS blob; a forward convolution whose own
+  // maxNumActOut differs could never use it (and, were the index tensor left unwritten for its sake, would have
+  // nothing to work from).  An inverse convolution derives its table from the index tensor whatever the sizes.
+  if (!m->inverse && r->maxNumActOut != m->maxNumActOut) {
+    setError("d3d_link_rulebook: maxNumActOut %d of the convolution, %d of the rulebook", m->maxNumActOut,
+             r->maxNumActOut);
     return D3D_ERR_BAD_ARG;
   }
   // tile masks are read by the kernels of layers with at least 32 (widened) input channels

@@ -11,6 +11,7 @@
 // on its stream.  Built on the public entry point d3d_enqueue only.
 #include <hip/hip_runtime.h>
 
+#include <cstring>
 #include <vector>
 
 #include "common.h"
@@ -92,6 +93,15 @@ int32_t d3d_schedule_add(d3d_schedule* s, d3d_plugin* plugin, const d3d_tensor_d
       lane >= static_cast<int32_t>(s->lanes.size())) {
     d3d::setError("schedule: bad step (null array, negative count or lane outside the schedule)");
     return D3D_ERR_BAD_ARG;
+  }
+  {
+    // the operators read fixed positions of the input arrays: a shorter array is a host out-of-bounds read
+    const char* type = d3d_plugin_type(plugin);
+    const int32_t need = !type ? 0 : (std::strncmp(type, "SPConvIdx", 9) == 0 ? 3 : (std::strcmp(type, "SPConvMM") == 0 ? 5 : 4));
+    if (nb_in < need) {
+      d3d::setError("schedule: %s reads %d inputs, step names %d", type ? type : "?", need, nb_in);
+      return D3D_ERR_BAD_ARG;
+    }
   }
   if (nb_out != d3d_num_outputs(plugin)) {
     d3d::setError("schedule: %s has %d outputs, step names %d", d3d_plugin_type(plugin), d3d_num_outputs(plugin), nb_out);

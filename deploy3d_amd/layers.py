@@ -53,8 +53,12 @@ class Rulebook:
 class SparseConvLayer:
     """One convolution: an SPConvMM plugin plus (for the first user of a key) an SPConvIdx plugin."""
 
-    def __init__(self, spec, weight, bias, max_num_act_out, dtype=torch.float16, device="cuda"):
+    def __init__(self, spec, weight, bias, max_num_act_out, dtype=torch.float16, device="cuda", extensions=True):
         self.spec = spec
+        # extensions=False: the operators as a caller of the reference's plugins would use them - no links between
+        # them, no persistent index tensor - so every enqueue fills its whole index tensor and every convolution
+        # derives its table from the tensor it is handed
+        self.extensions = extensions
         self.max_num_act_out = int(max_num_act_out)
         self.dtype = dtype
         self.device = device
@@ -63,7 +67,8 @@ class SparseConvLayer:
             spec["ksize"], spec["stride"], spec["padding"], spec["dilation"], (0,) * nd, self.max_num_act_out,
             spec["subm"], spec.get("transpose", False)))
         # the index tensor is allocated once below and written by this operator only
-        self.idx_plugin.set_option(OPT_PERSISTENT_INDEX, 1)
+        if extensions:
+            self.idx_plugin.set_option(OPT_PERSISTENT_INDEX, 1)
         self.mm_plugin = Plugin("SPConvMM", mm_blob(
             spec["ksize"], spec["cin"], spec["cout"], self.max_num_act_out, spec["subm"], spec.get("inverse", False),
             weight, bias, relu=spec.get("relu", False), act_scale_in=float(spec.get("s_in", 1.0)),
@@ -84,7 +89,7 @@ class SparseConvLayer:
                              device=self.device)
             self._idx_state = dict(cap=x.capacity, in_descs=in_descs, out_descs=out_descs, outs=outs, ws=ws)
             # a SubM rulebook on the outputs of a strided one reuses that operator's occupancy map
-            if self.spec["subm"]:
+            if self.spec["subm"] and self.extensions:
                 self.idx_plugin.link_coords(x.producer)
         st = self._idx_state
         self.idx_plugin.enqueue(st["in_descs"], st["out_descs"], [x.coors, x.num_act, None], st["outs"], st["ws"])
@@ -108,7 +113,8 @@ class SparseConvLayer:
         if self._mm_state is None or self._mm_state["in_rows"] != feats.shape[0] or self._mm_state["rb"] is not rb.plugin:
             in_descs = [TensorDesc.of_tensor(t) for t in (feats, num_in, num_out, rb.index, rb.num_index)]
             out_descs = self.mm_plugin.output_descs(in_descs)
-            self.mm_plugin.link_rulebook(rb.plugin)
+            if self.extensions:
+                self.mm_plugin.link_rulebook(rb.plugin)
             self.mm_plugin.configure(in_descs, out_descs)
             out = torch.empty(out_descs[0].shape(), dtype=self.dtype, device=self.device)
             self._mm_state = dict(in_rows=feats.shape[0], in_descs=in_descs, out_descs=out_descs, out=out, rb=rb.plugin)
@@ -134,24 +140,28 @@ class SparseBackbone:
     stage before it, which the convolutions need first.  The side streams fork from and join into the caller's current
     stream, so a forward pass can still be captured into one HIP graph (it then holds parallel branches).
 
+    ``extensions=False`` runs the operators as the reference's contract alone describes them (no links, no options).
+
     ``index_tensors=False`` tells the rulebook operators that nothing outside this runner reads their index tensors
     (``Rulebook.index`` is then unspecified): they write the tables the convolutions read and skip the compaction.
     """
 
     def __init__(self, layers, weights, capacities, dtype=torch.float16, device="cuda", overlap=True,
-                 index_tensors=True):
+                 index_tensors=True, extensions=True):
         self.specs = layers
-        self.layers = [SparseConvLayer(s, w, b, cap, dtype=dtype, device=device)
+        self.layers = [SparseConvLayer(s, w, b, cap, dtype=dtype, device=device, extensions=extensions)
                        for s, (w, b), cap in zip(layers, weights, capacities)]
         # every convolution reads the rulebook of the first layer that names its indice key: link them now, so
         # that already the first pass has the rulebook operators write the tables
         owner = {}
         for spec, lyr in zip(layers, self.layers):
-            lyr.mm_plugin.link_rulebook(owner.setdefault(spec["key"], lyr).idx_plugin)
+            first = owner.setdefault(spec["key"], lyr)
+            if extensions:
+                lyr.mm_plugin.link_rulebook(first.idx_plugin)
         # index_tensors=False: this runner is the only reader of the index tensors and its convolutions read the
         # linked tables, so the rulebook operators may leave the tensors unwritten (D3D_OPT_INDEX_UNUSED) - except
         # for a key that an inverse convolution uses, which works from the tensor
-        if not index_tensors:
+        if not index_tensors and extensions:
             inverse_keys = {spec["key"] for spec in layers if spec.get("inverse", False)}
             for key, lyr in owner.items():
                 if key not in inverse_keys:
@@ -164,12 +174,7 @@ class SparseBackbone:
         main = side = None
         if self.overlap:
             if self._side is None:  # strided rulebooks feed each other; SubM rulebooks hang off them
-                import os
-                if os.environ.get("D3D_ONE_SIDE"):
-                    one = torch.cuda.Stream()
-                    self._side = {False: one, True: one}
-                else:
-                    self._side = {False: torch.cuda.Stream(), True: torch.cuda.Stream()}
+                self._side = {False: torch.cuda.Stream(), True: torch.cuda.Stream()}
             main, side = torch.cuda.current_stream(), self._side
             fork = torch.cuda.Event()
             fork.record(main)

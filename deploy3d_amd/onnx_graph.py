@@ -360,6 +360,7 @@ class GraphExecutor:
                                           % (n.op_type, n.name or n.outputs))
         # graph edges: an SPConvMM reads the index tensor that an SPConvIdx node writes
         producer = {out: (i, j) for i, n in enumerate(self.nodes) for j, out in enumerate(n.outputs)}
+        linked = set()  # SPConvMM nodes whose link to the rulebook node was accepted
         for i, n in enumerate(self.nodes):
             p = self.plugins.get(i)
             if p is None:
@@ -379,7 +380,11 @@ class GraphExecutor:
                 if src is not None and src[1] == 0 and src[0] in self.plugins and \
                         self.plugins[src[0]].name.startswith("SPConvIdx") and \
                         producer.get(n.inputs[4]) == (src[0], 1):
-                    p.link_rulebook(self.plugins[src[0]])
+                    try:
+                        p.link_rulebook(self.plugins[src[0]])
+                        linked.add(i)
+                    except EngineError:
+                        pass  # kernel volume or maxNumActOut of the two nodes differ: this node derives its table
         # an index tensor that only linked forward convolutions read (not a graph output, no other consumer) need
         # not be written at all
         outputs = {v.name for v in model.outputs}
@@ -388,7 +393,7 @@ class GraphExecutor:
             if p is None or not p.name.startswith("SPConvIdx") or n.outputs[0] in outputs:
                 continue
             readers = [(j, m) for j, m in enumerate(self.nodes) if n.outputs[0] in m.inputs]
-            if readers and all(j in self.plugins and self.plugins[j].name == "SPConvMM" and len(m.inputs) >= 5 and
+            if readers and all(j in linked and self.plugins[j].name == "SPConvMM" and len(m.inputs) >= 5 and
                                m.inputs[3] == n.outputs[0] and m.inputs[4] == n.outputs[1] and
                                not self._inverse(m) for j, m in readers):
                 p.set_option(OPT_INDEX_UNUSED, 1)

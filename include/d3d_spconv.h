@@ -58,7 +58,11 @@ typedef struct d3d_plugin d3d_plugin;
  * trt/spconv/mm_trt.cu:222-227): the only constructor.  The blob is
  *   SPConvIdx{N}d: int32 kernelSize[N], stride[N], padding[N], dilation[N],
  *                  outPadding[N]; int32 maxNumActOut; u8 subM; u8 transpose
- *                  (packed; trt/spconv/index_trt.cu:39-50)
+ *                  (packed; trt/spconv/index_trt.cu:39-50).  Kernel sizes, strides and
+ *                  dilations must be positive: the reference's kernelSize == -1
+ *                  ("the whole extent", output extent 1: trt/spconv/geometry.h:129-131),
+ *                  which none of its own operators or tests produce, is refused with
+ *                  D3D_ERR_BAD_BLOB.
  *   SPConvMM:      int32 kernelVol, inChannels, outChannels, maxNumActOut;
  *                  u8 subM(ignored), inverse, withBias; fp32 W[kVol*Cin*Cout];
  *                  fp32 bias[Cout] iff withBias  (trt/spconv/mm_trt.cu:27-37, :61-68)

@@ -239,8 +239,38 @@ def test_schedule_bookkeeping_without_a_gpu():
     with pytest.raises(EngineError) as e:
         s.add(p, ins, outs[:1], [coors, num, None], [index])           # the operator has two outputs
     assert e.value.status == -3
+    with pytest.raises(EngineError) as e:
+        s.add(p, ins[:2], outs, [coors, num], [index, num_index])      # the operator reads three inputs
+    assert e.value.status == -3 and "reads 3 inputs" in str(e.value)
     with pytest.raises(EngineError):
         s.add(p, ins, outs, [coors, num, None], [index, num_index], after=[2])   # itself
     with pytest.raises(EngineError):
         s.add(p, ins, outs, [coors, num, None], [index, num_index], lane=1)
     assert len(s) == 2
+
+
+def test_a_link_between_nodes_of_different_sizes_is_refused():
+    """d3d_link_rulebook: the table a rulebook operator writes has maxNumActOut rows of ITS attribute blob
+    (reference: two independent blob fields, spconv_index.py:99 and spconv_mm.py:57).  A forward convolution with
+    another maxNumActOut could never use that table, so the link is refused; an inverse convolution, which always
+    derives its table from the index tensor, may link whatever the sizes; and so is one with another kernel volume."""
+    import numpy as np
+    from deploy3d_amd.spconv_mm import mm_blob
+    idx = Plugin("SPConvIdx3d", index_blob((3,) * 3, (2,) * 3, (1,) * 3, (1,) * 3, (0,) * 3, 512, False, False))
+    w = np.zeros((27, 4, 4), np.float32)
+    same = Plugin("SPConvMM", mm_blob((3, 3, 3), 4, 4, 512, False, False, w))
+    other = Plugin("SPConvMM", mm_blob((3, 3, 3), 4, 4, 256, False, False, w))
+    inverse = Plugin("SPConvMM", mm_blob((3, 3, 3), 4, 4, 256, False, True, w))
+    volume = Plugin("SPConvMM", mm_blob((1, 3, 3), 4, 4, 512, False, False, np.zeros((9, 4, 4), np.float32)))
+    for p in (other, volume):
+        with pytest.raises(EngineError) as e:
+            p.link_rulebook(idx)
+        assert e.value.status == -3
+    assert "maxNumActOut 256" in str(pytest.raises(EngineError, other.link_rulebook, idx).value)
+    # accepted links reserve device memory for the table: without a GPU they get as far as that (status -6), with
+    # one they succeed
+    for p in (same, inverse):
+        try:
+            p.link_rulebook(idx)
+        except EngineError as err:
+            assert err.status == -6

@@ -260,6 +260,31 @@ def test_duplicate_pairs_keep_the_highest_input(engine):
         check_close(got, ref, "float16")
 
 
+@pytest.mark.parametrize("cin,cout", [(32, 32), (128, 128), (16, 16)])
+def test_gather_rows_outside_the_input_are_no_neighbours(engine, cin, cout):
+    """A foreign index tensor whose gather row names no input row - negative other than -1, at or past the row
+    count, or so large that a row offset computed in 32 bits would wrap back inside the feature buffer (2^24 rows of
+    256 bytes) - contributes nothing: the derived table keeps -1 or existing rows only."""
+    n = 256
+    rng = np.random.default_rng(11)
+    feats = round_to(rng.standard_normal((n, cin)), "float16")
+    w = round_to(rng.standard_normal((27, cin, cout)) / np.sqrt(27 * cin), "float16")
+    row_len = 27 * (n + 128)
+    index = np.full((3, row_len), -1, np.int32)
+    bad = [n, n + 7, -5, (1 << 24) + 3, (1 << 25) + 1, np.iinfo(np.int32).max]
+    index[0, :3] = (5, 7, 9)
+    index[1, :3] = (5, 7, 5 + 64)
+    index[2, :3] = 13
+    index[0, 3:3 + len(bad)] = bad            # under the same tap, each feeding an output row of its own
+    index[1, 3:3 + len(bad)] = np.arange(100, 100 + len(bad))
+    index[2, 3:3 + len(bad)] = 13
+    keep = index.copy()
+    keep[:, 3:3 + len(bad)] = -1
+    ref = oracle.conv(feats, w, None, keep, 128, n, acc="f64")
+    got = _mm_on_index(index, 128, n, cin, cout, feats, w)
+    check_close(got, ref, "float16")
+
+
 @pytest.mark.parametrize("tile_rows", [128, 256, 512])
 @pytest.mark.parametrize("cin,cout", [(32, 64), (64, 64), (64, 128), (128, 128)])
 def test_mfma_tile_sizes(engine, monkeypatch, tile_rows, cin, cout):

@@ -1,6 +1,8 @@
 """The ONNX graph executor on the GPU: a graph of TRT_PluginV2 nodes run through deploy3d_amd.onnx_graph.GraphExecutor
-gives, bit for bit, what deploy3d_amd.layers.SparseBackbone gives for the layer table the graph was written from
-(which the other GPU tests hold against the oracle).  Parity unpinned by the reference, which has no graph fixture."""
+gives, bit for bit, what deploy3d_amd.layers.SparseBackbone gives for the layer table the graph was written from,
+and - the fixture graph and the config-3 graph - what the CPU oracle gives for that table (coordinates bit-exact
+after sorting, features within 2e-2 * rms).  The graph FILE itself is parity unpinned by the reference, which has
+no graph fixture."""
 import os
 import sys
 
@@ -26,6 +28,22 @@ def _same(y, out, model):
     assert torch.equal(feats, y.feats)
 
 
+def _against_the_oracle(out, model, cfg, last):
+    """The executor's sparse outputs against the CPU oracle run over the layer table the graph was written from:
+    the same coordinates (bit for bit after sorting both by coordinate), features within 2e-2 * rms (fp16 storage,
+    fp32 accumulation on the GPU, fp64 in the oracle)."""
+    import chain
+    ref = chain.oracle_chain(cfg)[last]
+    feats, coors, num = (out[v.name] for v in model.outputs[:3])
+    n = int(num.item())
+    assert n == len(ref["coords"])
+    c_gpu, f_gpu = chain.sort_rows(coors[:n].cpu().numpy(), feats[:n].float().cpu().numpy())
+    c_ref, f_ref = chain.sort_rows(ref["coords"], ref["feats"])
+    assert np.array_equal(c_gpu, c_ref)
+    rms = float(np.sqrt(np.mean(f_ref.astype(np.float64) ** 2)))
+    assert rms > 0 and np.abs(f_gpu.astype(np.float64) - f_ref).max() <= 2e-2 * rms
+
+
 def test_fixture_file_runs_like_the_layer_table(engine):
     import make_onnx_graph
     from deploy3d_amd import layers, onnx_graph, synth
@@ -38,6 +56,10 @@ def test_fixture_file_runs_like_the_layer_table(engine):
     out = ex.run(**_graph_inputs(x, make_onnx_graph.GRID))
     torch.cuda.synchronize()
     _same(y, out, ex.model)
+    # ... and like the CPU oracle on that table: the executor's result does not rest on the engine agreeing with itself
+    cfg = dict(dtype="float16", coords=coords, feats=feats, grid=list(make_onnx_graph.GRID), layers=specs,
+               weights=weights)
+    _against_the_oracle(out, ex.model, cfg, specs[-1]["name"])
 
 
 @pytest.mark.parametrize("config,n", [(3, 12000), (5, 20000)])
@@ -63,6 +85,8 @@ def test_whole_configurations_and_graph_capture(engine, config, n):
         torch.cuda.synchronize()
         _same(y, out, ex.model)
         assert torch.equal(out["bev"], bev)
+    if config == 3:  # the final tensor of the whole backbone against the CPU oracle
+        _against_the_oracle(out, ex.model, cfg, specs[-1]["name"])
     # the same graph through the native schedule: one call per pass, rulebook nodes on lanes of their own
     if config == 3:
         for live in (n // 3, n):

@@ -115,3 +115,55 @@ def test_static_scratch_limits(engine):
         mm.enqueue(ins, outs, [x, num, num, idx, num], [torch.empty((64, 16), dtype=torch.float16, device="cuda")],
                    "static")
     assert e.value.status == -1
+
+
+def test_static_enqueue_allocates_nothing(engine):
+    """The entry point's promise itself: free device memory is the same before and after static calls (operators made
+    and tensors allocated beforehand), also for a strided operator that keeps a map for a linked submanifold
+    operator and has the persistent-index option set (both would otherwise make the library allocate on first use);
+    and the calls can be recorded into a HIP graph in the capture mode that refuses allocation, and replayed."""
+    from deploy3d_amd import Plugin, TensorDesc
+    from deploy3d_amd.plugin import OPT_PERSISTENT_INDEX
+    from deploy3d_amd.spconv_index import index_blob
+    grid, n = (12, 96, 96), 6000
+    rng = np.random.default_rng(75)
+    coords = random_cloud(rng, n, grid, 1)
+    strided = Plugin("SPConvIdx3d", index_blob((3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1), (0, 0, 0), 4 * n, False, False))
+    subm = Plugin("SPConvIdx3d", index_blob((3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), (0, 0, 0), 4 * n, True, False))
+    strided.set_option(OPT_PERSISTENT_INDEX, 1)
+    subm.link_coords(strided)
+    c = torch.from_numpy(coords).cuda()
+    num = torch.tensor([n], dtype=torch.int32, device="cuda")
+    ins = [TensorDesc.of_tensor(c), TensorDesc.of_tensor(num), TensorDesc.of((1, 0) + grid, torch.int32)]
+    outs = strided.output_descs(ins)
+    bufs = [torch.full(d.shape(), 7, dtype=torch.int32, device="cuda") if 0 not in d.shape() else None for d in outs]
+    ins2 = [TensorDesc.of_tensor(bufs[2]), TensorDesc.of_tensor(bufs[3]), TensorDesc.of((1, 0, 6, 48, 48), torch.int32)]
+    outs2 = subm.output_descs(ins2)
+    bufs2 = [torch.full(d.shape(), 7, dtype=torch.int32, device="cuda") for d in outs2]
+    want = _index_outputs(Plugin("SPConvIdx3d", index_blob((3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1), (0, 0, 0),
+                                                           4 * n, False, False)), coords, n, grid, None)
+
+    def both():
+        strided.enqueue(ins, outs, [c, num, None], bufs, "static")
+        subm.enqueue(ins2, outs2, [bufs[2], bufs[3], None], bufs2, "static")
+
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    both()
+    both()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.equal(bufs[0], want[0]) and torch.equal(bufs[1], want[1])
+    first = [b.clone() for b in bufs2]
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream, capture_error_mode="global"):
+            both()
+        for b in bufs2:
+            b.fill_(7)
+        graph.replay()
+        graph.replay()
+    stream.synchronize()
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(first, bufs2))
