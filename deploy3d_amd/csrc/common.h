@@ -157,6 +157,8 @@ struct ConvArgs {
   int64_t nbrPitch;       // row pitch of nbr in elements; 0 = outRows
   int tapMirror;          // the table is indexed by the mirrored tap (a SubM rulebook's input-major table, see rbCompact)
   const unsigned long long* tileMasks;  // optional [ceil(outRows / 64)]: bit t set iff any of rows 64i..64i+63 has tap t
+  const int32_t* numActOut;  // device int32 or null: live output rows (tiles past them only take their bias; the
+                          // kernels balance the live ones over the chip)
   const void* zeros;      // device, >= 512 zero bytes: the row that absent neighbours gather
   int relu;
   int tileRows;           // 0 = choose; else rows per workgroup of the weight-streaming MFMA kernel (128, 256, 512)

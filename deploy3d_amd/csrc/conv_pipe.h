@@ -42,7 +42,7 @@ __global__ void __launch_bounds__(64 * WAVES)
 convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
          const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror,
          const unsigned long long* __restrict__ tileMasks, int kVol, int64_t inRows, int64_t outRows, int relu,
-         int tileBlocks, int xcdShift) {
+         int tileBlocks, int xcdShift, const int32_t* __restrict__ numActOut) {
   constexpr int THREADS = 64 * WAVES;
   constexpr int ES = static_cast<int>(sizeof(T));
   constexpr int CS = CIN > 64 ? 64 : CIN;                      // input channels per step; a tap takes KS steps
@@ -96,24 +96,20 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
     idxRow[i] = static_cast<uint32_t>(wave * WM + (p % GL) * RPI + p / GL);
   }
 
-  // ---- this workgroup's tiles: XCD x serves the x-th contiguous part of the tiles (neighbouring tiles gather
-  // many of the same rows: they should meet behind one L2); inside it, workgroups take tiles round robin ----
-  const int nXcd = 1 << xcdShift;
-  const int perXcd = (tileBlocks + nXcd - 1) >> xcdShift;
-  const int xcd = blockIdx.x & (nXcd - 1);
+  // ---- this workgroup's tiles: XCD x serves the x-th contiguous part of the tiles that hold live rows
+  // (neighbouring tiles gather many of the same rows: they should meet behind one L2) and its share of the tiles
+  // past the live rows; inside an XCD, workgroups take tiles round robin ----
+  const TileOrder order(tileBlocks, static_cast<int>((liveOutRows(numActOut, outRows) + TM - 1) / TM), xcdShift,
+                        blockIdx.x & ((1 << xcdShift) - 1));
   const int firstLocal = blockIdx.x >> xcdShift, strideLocal = gridDim.x >> xcdShift;
-  int nMine = 0;
-  if (firstLocal < perXcd) {
-    int lastLocal = perXcd - 1;
-    if (xcd * perXcd + lastLocal >= tileBlocks) lastLocal = tileBlocks - 1 - xcd * perXcd;
-    if (lastLocal >= firstLocal) nMine = (lastLocal - firstLocal) / strideLocal + 1;
-  }
+  const int nMine = firstLocal < order.count() ? (order.count() - 1 - firstLocal) / strideLocal + 1 : 0;
   if (nMine <= 0) return;                                // workgroup-uniform
-  auto tileAt = [&](int pos) __attribute__((always_inline)) { return xcd * perXcd + firstLocal + pos * strideLocal; };
+  auto tileAt = [&](int pos) __attribute__((always_inline)) { return order.tile(firstLocal + pos * strideLocal); };
   const unsigned long long allTaps = kVol >= 64 ? ~0ull : ((1ull << kVol) - 1ull);
   // taps of the workgroup's pos-th tile; a tile without any tap still takes one step (tap 0: all rows absent)
   auto maskAt = [&](int pos) __attribute__((always_inline)) -> unsigned long long {
     if (pos >= nMine) return 0ull;
+    if (!order.live(firstLocal + pos * strideLocal)) return 1ull;   // no live row: one step of absent neighbours
     unsigned long long m = allTaps;
     if (tileMasks) {
       const unsigned long long* p = tileMasks + static_cast<int64_t>(tileAt(pos)) * PER;
@@ -395,7 +391,7 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((convPipe<T, CIN, COUT, MT, WAVES>), dim3(static_cast<unsigned>(blocks)), dim3(64 * WAVES),
                      lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
                      static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, pitch, a.tapMirror, a.tileMasks, a.kVol,
-                     a.inRows, a.outRows, a.relu, tiles, chip.xcdShift);
+                     a.inRows, a.outRows, a.relu, tiles, chip.xcdShift, a.numActOut);
   return D3D_OK;
 }
 

@@ -1007,6 +1007,7 @@ struct MMPlugin final : d3d_plugin {
     a.requantM = dtype == D3D_INT8 ? static_cast<const float*>(dev->requantM.ptr) : nullptr;
     a.nbr = nbr;
     a.tileMasks = masks;
+    a.numActOut = static_cast<const int32_t*>(inputs[2]);
     a.relu = relu ? 1 : 0;
     a.zeros = zeros;
     if (const char* e = debugEnv("D3D_CONV_PIPE")) a.pipe = e[0] == '0' ? -1 : 0;
