@@ -77,30 +77,6 @@ template <> struct Mfma<int8_t> {
   }
 };
 
-// Fragment type per K step: 8 elements (16 bytes) when CIN >= 32, else 4.
-template <int CIN> struct Frag { using type = u32x4; };
-template <> struct Frag<16> { using type = u32x2; };
-
-// Weights live in LDS in the same fragment-major order as in global memory:
-// fragment (kk, n) of a tap is 64 consecutive lanes' worth of data, so a
-// wavefront read is one contiguous, conflict-free sweep.
-//
-// RESIDENT = true : the weights of ALL taps fit in LDS.  They are loaded once
-//   in the prologue and shared by up to 16 wavefronts; after that every
-//   wavefront runs alone (its own list of the taps that occur among its rows,
-//   no barriers).
-// RESIDENT = false: one tap's weights at a time, double-buffered.  The slice of
-//   tap t+1 travels global -> registers -> idle LDS buffer while tap t
-//   multiplies; one barrier per tap.  The weights are requested before the
-//   rows, because the vector-memory counter retires in order: waiting for a
-//   weight slice must not drain the younger gathers behind it.
-// Either way three register sets of gathered rows rotate, so the gathers of
-// taps t+1 and t+2 are in flight while tap t multiplies.  The rotation is
-// written out as three pipeline steps per loop iteration, with no branch
-// between them (the tap list is padded to a multiple of three with null taps
-// whose rows all come from the zero row), so that the compiler can neither
-// sink a gather towards its use nor has to copy a register set that is still
-// being loaded.
 // Which tiles (or row groups) a persistent workgroup serves, in which order.  Workgroups are dealt to the XCDs
 // round-robin; XCD x serves the x-th contiguous part of the tiles that hold LIVE rows (neighbouring tiles gather
 // many of the same rows: they meet behind one L2), and every n-th of the tiles past the live rows, which only
@@ -134,6 +110,30 @@ __device__ __forceinline__ int64_t liveOutRows(const int32_t* numActOut, int64_t
   return n < 0 ? 0 : (n > outRows ? outRows : n);
 }
 
+// Fragment type per K step: 8 elements (16 bytes) when CIN >= 32, else 4.
+template <int CIN> struct Frag { using type = u32x4; };
+template <> struct Frag<16> { using type = u32x2; };
+
+// Weights live in LDS in the same fragment-major order as in global memory:
+// fragment (kk, n) of a tap is 64 consecutive lanes' worth of data, so a
+// wavefront read is one contiguous, conflict-free sweep.
+//
+// RESIDENT = true : the weights of ALL taps fit in LDS.  They are loaded once
+//   in the prologue and shared by up to 16 wavefronts; after that every
+//   wavefront runs alone (its own list of the taps that occur among its rows,
+//   no barriers).
+// RESIDENT = false: one tap's weights at a time, double-buffered.  The slice of
+//   tap t+1 travels global -> registers -> idle LDS buffer while tap t
+//   multiplies; one barrier per tap.  The weights are requested before the
+//   rows, because the vector-memory counter retires in order: waiting for a
+//   weight slice must not drain the younger gathers behind it.
+// Either way three register sets of gathered rows rotate, so the gathers of
+// taps t+1 and t+2 are in flight while tap t multiplies.  The rotation is
+// written out as three pipeline steps per loop iteration, with no branch
+// between them (the tap list is padded to a multiple of three with null taps
+// whose rows all come from the zero row), so that the compiler can neither
+// sink a gather towards its use nor has to copy a register set that is still
+// being loaded.
 template <class T, int CIN, int COUT, int MT, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES)
 convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,

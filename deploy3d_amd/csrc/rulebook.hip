@@ -286,22 +286,15 @@ __device__ __forceinline__ bool tapTarget(const RbGeom& g, const int c[5], const
   return ok;
 }
 
-// Pairs per tap are kept as kTotalSlots partial sums, totals[tap * kTotalSlots + slot]: atomics on one address are
-// performed one after the other (about 18 ns each across the XCDs), and a pass whose every workgroup adds to the
-// one word of its tap spends longer queueing there than working (1 400 workgroups: 25 us).
+// Words per tap of the workspace area behind the pair counts (the hash path keeps its owned-output counts per
+// tap there; the pair counts themselves need no per-tap totals: the compaction sums the rows of counts).  Atomics
+// on one address are performed one after the other (about 18 ns each across the XCDs), device-wide atomics run
+// at a few per nanosecond in all: passes that every workgroup ended with a handful of them spent more time there
+// than on their loads and stores.
 constexpr int kTotalSlots = 8;
 
-// Pairs per (tap, block of 256 or 1024 inputs): at most 1024, kept in 16 bits so that a row of counts is short.
+// Pairs per (tap, block of 256 or 512 inputs), kept in 16 bits so that a row of counts is short.
 typedef uint16_t RbCount;
-
-__device__ __forceinline__ uint32_t tapPairs(const uint32_t* __restrict__ totals, int tap) {
-  const uint4 a = *reinterpret_cast<const uint4*>(totals + tap * kTotalSlots);
-  const uint4 b = *reinterpret_cast<const uint4*>(totals + tap * kTotalSlots + 4);
-  return a.x + a.y + a.z + a.w + b.x + b.y + b.z + b.w;
-}
-__device__ __forceinline__ uint32_t tapSegment(const uint32_t* __restrict__ totals, int tap) {
-  return (tapPairs(totals, tap) + (kSegment - 1)) & ~static_cast<uint32_t>(kSegment - 1);
-}
 
 // Publishes the number of flagged items of this workgroup for its tap in cnt (row pitch nBlocks) and, when `totals` is
 // given, adds it to the per-tap sums there (`slots` partial sums per tap).
@@ -313,6 +306,16 @@ __device__ __forceinline__ void publishCount(uint32_t mine, uint32_t* scratch, C
     cnt[static_cast<size_t>(blockIdx.y) * nBlocks + blockIdx.x] = static_cast<Count>(total);
     if (total && totals) atomicAdd(&totals[blockIdx.y * slots + blockIdx.x % slots], total);
   }
+}
+
+// Pairs per (tap, 256 inputs) of the passes that run one workgroup per (chunk of 1024 inputs, tap): a wavefront's
+// lanes hold 256 consecutive inputs, so every wavefront stores the count of its own block (row pitch `pitch`).
+__device__ __forceinline__ void publishWaveCounts(uint32_t mine, RbCount* cnt, uint32_t pitch) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mine += __shfl_down(mine, off, 64);
+  if ((threadIdx.x & 63) == 0)
+    cnt[static_cast<size_t>(blockIdx.y) * pitch + blockIdx.x * (kRbThreads / 64) + (threadIdx.x >> 6)] =
+        static_cast<RbCount>(mine);
 }
 
 // SubM: coordinate -> row map (reference: setSubMHashKernel, index.cu:174-182)
@@ -333,7 +336,6 @@ __global__ void __launch_bounds__(kRbThreads)
 rbSubmProbe(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restrict__ numActIn, int64_t cap,
             int64_t pitch, const unsigned long long* __restrict__ table, uint32_t mask, uint32_t* __restrict__ staging,
             RbCount* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
-  __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
   const int tap = blockIdx.y;
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
@@ -356,7 +358,7 @@ rbSubmProbe(RbGeom g, const int32_t* __restrict__ coors, const int32_t* __restri
     if (first < n) *reinterpret_cast<uint4*>(staging + static_cast<int64_t>(tap) * pitch + first) =
         make_uint4(row[0], row[1], row[2], row[3]);
   }
-  publishCount(found, scratch, cnt, nBlocks, totals, kTotalSlots);
+  publishWaveCounts(found, cnt, nBlocks);
 }
 
 // ---------------------------------------------------------------------------
@@ -491,7 +493,6 @@ __global__ void __launch_bounds__(kRbThreads)
 rbConvResolve(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, const uint32_t* __restrict__ ids,
               uint32_t* __restrict__ staging, int32_t maxNumActOut, RbCount* __restrict__ cnt, uint32_t nBlocks,
               uint32_t* totals) {
-  __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
   const int tap = blockIdx.y;
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
@@ -512,7 +513,7 @@ rbConvResolve(const int32_t* __restrict__ numActIn, int64_t cap, int64_t pitch, 
     }
     *cell = make_uint4(v[0], v[1], v[2], v[3]);
   }
-  publishCount(found, scratch, cnt, nBlocks, totals, kTotalSlots);
+  publishWaveCounts(found, cnt, nBlocks);
 }
 
 // ---------------------------------------------------------------------------
@@ -570,7 +571,7 @@ __device__ __forceinline__ uint32_t countsBelow(const uint4& v, uint32_t b0, uin
 
 // MIRROR: the table is that of a SubM rulebook with "same" padding (see below).  SKIP: the index tensor is left
 // unwritten (nothing reads it): what remains is numIndex and, where inputs were not in rank order, the ranks in
-// the mirrored table turned into rows.  SHIFT: log2 of the inputs per entry of cnt (8, 9 or 10); a wavefront
+// the mirrored table turned into rows.  SHIFT: log2 of the inputs per entry of cnt (8 or 9); a wavefront
 // compacts exactly one such block, 1 << (SHIFT - 6) consecutive inputs per lane, so its write position is the
 // workgroup's plus the counts of the workgroup's earlier blocks - after the one barrier behind the sums the
 // wavefronts run on their own, each as soon as its own staging entries have arrived.
@@ -1251,7 +1252,6 @@ bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* 
         const uint32_t* __restrict__ perm, const uint32_t* __restrict__ permShuffled, int32_t maxNumActOut,
         uint32_t* __restrict__ staging, RbCount* __restrict__ cnt, uint32_t nBlocks, uint32_t* totals) {
   const BmRecord* __restrict__ records = recRef.get();
-  __shared__ uint32_t scratch[kRbThreads / 64];
   const int n = liveCount(numActIn, cap);
   const int tap = blockIdx.y;
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kRbChunk + threadIdx.x * kRbItems;
@@ -1282,7 +1282,7 @@ bmProbe(RbGeom g, BlockMap m, const int32_t* __restrict__ coors, const int32_t* 
     if (first < n) *reinterpret_cast<uint4*>(staging + static_cast<int64_t>(tap) * pitch + first) =
         make_uint4(row[0], row[1], row[2], row[3]);
   }
-  publishCount(found, scratch, cnt, nBlocks, totals, kTotalSlots);
+  publishWaveCounts(found, cnt, nBlocks);
 }
 
 // ---------------------------------------------------------------------------
@@ -2009,7 +2009,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
   bool skipIndex = false;                     // set below when side.skipIndex can be honoured
   bool directScatter = false;                 // the probe pass writes the scattered table itself
   bool needReset = true;                      // a reset pass opens the build
-  int cntShift = 10;                          // log2 of the inputs one entry of cnt covers
+  int cntShift = 8;                           // log2 of the inputs one entry of cnt covers
   unsigned long long* compactMasks = masks;   // null when the probe pass writes the masks itself
   const uint32_t* compactPerm = nullptr;      // block-map SubM: staging holds ranks, rows = perm[rank] when shuffled
   const uint32_t* compactPermFlag = nullptr;
@@ -2199,8 +2199,7 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
 #define D3D_LAUNCH_COMPACT_SHIFT(MIRROR, SKIP)                        \
   do {                                                                \
     if (cntShift == 8) D3D_LAUNCH_COMPACT(MIRROR, SKIP, 8);           \
-    else if (cntShift == 9) D3D_LAUNCH_COMPACT(MIRROR, SKIP, 9);      \
-    else D3D_LAUNCH_COMPACT(MIRROR, SKIP, 10);                        \
+    else D3D_LAUNCH_COMPACT(MIRROR, SKIP, 9);                         \
   } while (0)
   if (skipIndex) {
     if (mirror) D3D_LAUNCH_COMPACT_SHIFT(true, true); else D3D_LAUNCH_COMPACT_SHIFT(false, true);
