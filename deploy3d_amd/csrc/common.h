@@ -147,6 +147,7 @@ struct ConvArgs {
   const void* in;
   const void* inNarrow;   // the rows as the caller passed them, cinNarrow channels wide (in may be a widened copy)
   int cinNarrow;
+  int rowChannels;        // channels a row of `in` stores when fewer than cin (the kernel reads the rest as zeros); 0 = cin
   void* out;
   const float* weightsF32;  // device fp32 [kVol, cin, cout], values already rounded to the storage type
   const void* weightsMfma;  // device storage-type, MFMA fragment-major (see MMPlugin::configure) or null
@@ -182,6 +183,9 @@ bool convUsesMfma(int32_t dtype, int cin, int cout);
 // Input-channel count the MFMA path would run a layer at (the next of 16/32/64/128 for 2-byte types when the
 // output channels qualify), else cin itself; and the kernel that widens rows to it with zero channels.
 int paddedMfmaChannels(int32_t dtype, int cin, int cout);
+// True when the layer's kernel reads rows of `cin` stored channels as they are although its MFMA contracts
+// paddedMfmaChannels() of them (ConvArgs::rowChannels): no widened copy of the input is needed.
+bool convReadsNarrowRows(int32_t dtype, int kVol, int cin, int cout);
 int32_t launchPadRows(const void* in, int64_t rows, int inBytes, int outBytes, void* out, hipStream_t stream);
 
 // Sparse rows -> dense [B, C, Z, Y, X] map (densify.hip).  The workspace holds one int32 per cell.

@@ -293,7 +293,7 @@ padRows(const uint8_t* __restrict__ in, int64_t rows, int inBytes, int outBytes,
 }  // namespace
 
 bool convUsesMfma(int32_t dtype, int cin, int cout) {
-  if (dtype == D3D_INT8) return (cin == 32 || cin == 64 || cin == 128) && isMfmaChannels(cout) && cin * cout >= 1024;
+  if (dtype == D3D_INT8) return (cin == 32 || cin == 64 || cin == 128) && isMfmaChannels(cout);
   return (dtype == D3D_HALF || dtype == D3D_BF16) && isMfmaChannels(cin) && isMfmaChannels(cout);
 }
 
@@ -304,9 +304,9 @@ int paddedMfmaChannels(int32_t dtype, int cin, int cout) {
     while (c < cin) c *= 2;
     return c;
   }
-  if (dtype == D3D_INT8) {  // the int8 MFMA contracts at least 32 channels; a step's weights fill at least 1 KiB
+  if (dtype == D3D_INT8) {  // the int8 MFMA contracts at least 32 channels
     int c = 32;
-    while (c < cin || c * cout < 1024) c *= 2;
+    while (c < cin) c *= 2;
     return c <= 128 ? c : cin;
   }
   return cin;

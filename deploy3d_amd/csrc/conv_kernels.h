@@ -5,6 +5,7 @@
 #include <hip/hip_fp16.h>
 
 #include <atomic>
+#include <type_traits>
 
 #include "common.h"
 
@@ -313,22 +314,27 @@ convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
 // Small layers: the weights of ALL taps fit in LDS.  A workgroup loads them once and then lives on: each of
 // its wavefronts walks, on its own, over groups of 16 output rows (group index strided by the number of
 // wavefronts in the grid), with a private slice of the neighbour table, its own list of the taps that occur
-// in the group, and no barrier after the weight load.
-template <class T, int CIN, int COUT, int WAVES>
+// in the group, and no barrier after the weight load.  CROW < CIN: the rows of `in` store CROW channels only and
+// the lanes that would read the others multiply zeros (their weights are zero rows as well).
+template <class T, int CIN, int COUT, int WAVES, int CROW = CIN>
 __global__ void __launch_bounds__(64 * WAVES)
 convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf,
-                 const float* __restrict__ bias, const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror,
-                 const T* __restrict__ zeros, int kVol, int64_t inRows, int64_t outRows, int relu, int groups,
-                 int xcdShift, const int32_t* __restrict__ numActOut) {
+                 const float* __restrict__ bias, const float* __restrict__ requantM, const int32_t* __restrict__ nbr,
+                 int64_t nbrPitch, int tapMirror, const T* __restrict__ zeros, int kVol, int64_t inRows,
+                 int64_t outRows, int relu, int groups, int xcdShift, const int32_t* __restrict__ numActOut) {
   constexpr int THREADS = 64 * WAVES;
   constexpr int MT = 1;
   constexpr int NT = COUT / 16;
-  constexpr int KSTEP = CIN >= 32 ? 32 : 16;
+  constexpr int ES = static_cast<int>(sizeof(T));              // 2: fp16 / bf16, 1: int8
+  constexpr bool WIDE = CIN * ES >= 64;                        // 16-byte operand fragments (else 8-byte)
+  constexpr int KSTEP = (WIDE ? 64 : 32) / ES;                 // channels one MFMA contracts
   constexpr int KK = CIN / KSTEP;
   constexpr int KG = KSTEP / 4;
   constexpr int WFRAGS = KK * NT * 64;
-  constexpr int WCHUNKS = CIN * COUT / 8;
-  using F = typename Frag<CIN>::type;
+  constexpr int WCHUNKS = CIN * COUT * ES / 16;
+  using F = typename std::conditional<WIDE, u32x4, u32x2>::type;
+  using Acc = typename Mfma<T>::Acc;
+  static_assert(CIN % KSTEP == 0 && (CROW == CIN || (KK == 1 && CROW % KG == 0)), "whole MFMA steps");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   F* wLds = reinterpret_cast<F*>(smem);                                              // [kVol][WFRAGS]
@@ -347,7 +353,8 @@ convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restr
 
   auto gatherRows = [&](int tap, F (&dst)[MT][KK]) __attribute__((always_inline)) {
     const int32_t src = tap < 0 ? -1 : nb[tap * 16 + r16];
-    const T* rowPtr = (src < 0 ? zeros : in + static_cast<size_t>(src) * CIN) + kgrp * KG;
+    const T* rowPtr = (src < 0 || kgrp * KG >= CROW ? zeros : in + static_cast<size_t>(src) * CROW + kgrp * KG);
+    if constexpr (CROW == CIN) rowPtr = (src < 0 ? zeros : in + static_cast<size_t>(src) * CIN) + kgrp * KG;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) dst[0][kk] = *reinterpret_cast<const F*>(rowPtr + kk * KSTEP);
   };
@@ -392,16 +399,16 @@ convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restr
       return wLds + static_cast<size_t>(tap < 0 ? 0 : tap) * WFRAGS;  // a null tap multiplies zero rows
     };
 
-    float4v acc[NT];
+    Acc acc[NT];
 #pragma unroll
-    for (int n = 0; n < NT; ++n) acc[n] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int n = 0; n < NT; ++n) acc[n] = Acc{0, 0, 0, 0};
     auto multiply = [&](const F* wTap, const F (&rows)[MT][KK]) __attribute__((always_inline)) {
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
         for (int n = 0; n < NT; ++n) {
           const F wfrag = wTap[(kk * NT + n) * 64 + lane];
-          if constexpr (CIN >= 32) {
+          if constexpr (WIDE) {
             acc[n] = Mfma<T>::k32(wfrag, rows[0][kk], acc[n]);
           } else {
             acc[n] = Mfma<T>::k16(wfrag, rows[0][kk], acc[n]);
@@ -437,14 +444,28 @@ convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restr
 #pragma unroll
       for (int n = 0; n < NT; ++n) {
         const int col = n * 16 + kgrp * 4;
-        float v[4];
+        if constexpr (ES == 1) {
+          // int8: t = float(acc) * m[c]; t += bq[c]; round to nearest even; clamp (lo = 0 with the fused ReLU)
+          uint32_t packed = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          v[j] = acc[n][j] + (bias ? bias[col + j] : 0.f);
-          if (relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
+          for (int j = 0; j < 4; ++j) {
+            float t = static_cast<float>(acc[n][j]) * requantM[col + j];
+            t = t + (bias ? bias[col + j] : 0.f);
+            float q = __builtin_rintf(t);
+            q = __builtin_fminf(127.f, __builtin_fmaxf(relu ? 0.f : -128.f, q));
+            packed |= (static_cast<uint32_t>(static_cast<int>(q)) & 0xFFu) << (8 * j);
+          }
+          *reinterpret_cast<uint32_t*>(out + static_cast<size_t>(row) * COUT + col) = packed;
+        } else {
+          float v[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v[j] = acc[n][j] + (bias ? bias[col + j] : 0.f);
+            if (relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
+          }
+          T packed[4] = {static_cast<T>(v[0]), static_cast<T>(v[1]), static_cast<T>(v[2]), static_cast<T>(v[3])};
+          *reinterpret_cast<u32x2*>(out + static_cast<size_t>(row) * COUT + col) = __builtin_bit_cast(u32x2, packed);
         }
-        T packed[4] = {static_cast<T>(v[0]), static_cast<T>(v[1]), static_cast<T>(v[2]), static_cast<T>(v[3])};
-        *reinterpret_cast<u32x2*>(out + static_cast<size_t>(row) * COUT + col) = __builtin_bit_cast(u32x2, packed);
       }
     }
   }
@@ -919,12 +940,12 @@ int32_t launchMfmaTile(const ConvArgs& a, hipStream_t stream) {
   return D3D_OK;
 }
 
-template <class T, int CIN, int COUT>
+template <class T, int CIN, int COUT, int CROW = CIN>
 int32_t launchMfmaResident(const ConvArgs& a, hipStream_t stream) {
   constexpr int WAVES = 16;
   const size_t lds = static_cast<size_t>(a.kVol) * CIN * COUT * sizeof(T) + static_cast<size_t>(WAVES) * a.kVol * 16 * 4;
   static std::atomic<size_t> granted{64 * 1024};
-  const int32_t rc = grantLds(&convMfmaResident<T, CIN, COUT, WAVES>, lds, &granted);
+  const int32_t rc = grantLds(&convMfmaResident<T, CIN, COUT, WAVES, CROW>, lds, &granted);
   if (rc != D3D_OK) return rc;
   const int groups = static_cast<int>((a.outRows + 15) / 16);
   // persistent workgroups: as many as fit on the CUs at this LDS footprint, but no more than there is work
@@ -937,11 +958,11 @@ int32_t launchMfmaResident(const ConvArgs& a, hipStream_t stream) {
   const int needed = (groups + WAVES - 1) / WAVES;
   if (blocks > needed) blocks = (needed + nXcd - 1) / nXcd * nXcd;
   if (blocks < nXcd) blocks = nXcd;
-  hipLaunchKernelGGL((convMfmaResident<T, CIN, COUT, WAVES>), dim3(static_cast<unsigned>(blocks)), dim3(64 * WAVES),
+  hipLaunchKernelGGL((convMfmaResident<T, CIN, COUT, WAVES, CROW>), dim3(static_cast<unsigned>(blocks)), dim3(64 * WAVES),
                      lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
-                     static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, a.nbrPitch > 0 ? a.nbrPitch : a.outRows,
-                     a.tapMirror, static_cast<const T*>(a.zeros), a.kVol, a.inRows, a.outRows, a.relu, groups,
-                     chip.xcdShift, a.numActOut);
+                     static_cast<const T*>(a.weightsMfma), a.bias, a.requantM, a.nbr,
+                     a.nbrPitch > 0 ? a.nbrPitch : a.outRows, a.tapMirror, static_cast<const T*>(a.zeros), a.kVol,
+                     a.inRows, a.outRows, a.relu, groups, chip.xcdShift, a.numActOut);
   return D3D_OK;
 }
 
@@ -1064,8 +1085,35 @@ int32_t launchMfma(const ConvArgs& a, hipStream_t stream) {
   return D3D_ERR_UNSUPPORTED;
 }
 
+// Weights of every tap resident in LDS (register gathers, no barriers): what the 32-channel int8 layers of few
+// output channels run, like the 16-channel layers in two-byte types - their rows are as many bytes.
+inline bool int8ResidentFits(int kVol, int cin, int cout) {
+  const size_t allTaps = static_cast<size_t>(kVol) * cin * cout;
+  return allTaps <= 56 * 1024 && kVol <= 128 && allTaps + static_cast<size_t>(16) * kVol * 16 * 4 <= kLdsLimit;
+}
+
+template <int CIN, int COUT, int CROW = CIN>
+int32_t launchInt8Resident(const ConvArgs& a, hipStream_t stream) {
+  if (int8ResidentFits(a.kVol, CIN, COUT)) return launchMfmaResident<int8_t, CIN, COUT, CROW>(a, stream);
+  return D3D_ERR_UNSUPPORTED;
+}
+
 template <int CIN>
 int32_t launchInt8Cout(const ConvArgs& a, hipStream_t stream) {
+  if constexpr (CIN == 32) {
+    int32_t rc = D3D_ERR_UNSUPPORTED;
+    if (a.rowChannels == 16) {  // rows of 16 stored channels: only the resident kernel reads them as they are
+      if (a.cout == 16) return launchInt8Resident<32, 16, 16>(a, stream);
+      if (a.cout == 32) return launchInt8Resident<32, 32, 16>(a, stream);
+      return D3D_ERR_UNSUPPORTED;
+    }
+    if (a.staged == 0) {
+      if (a.cout == 16) rc = launchInt8Resident<32, 16>(a, stream);
+      if (a.cout == 32 && a.tileMasks == nullptr) rc = launchInt8Resident<32, 32>(a, stream);
+      if (a.cout == 64 && a.tileMasks == nullptr) rc = launchInt8Resident<32, 64>(a, stream);
+    }
+    if (rc != D3D_ERR_UNSUPPORTED) return rc;
+  }
   switch (a.cout) {
     case 16: if constexpr (CIN * 16 >= 1024) return launchStaged<int8_t, CIN, 16>(a, stream); break;
     case 32: return launchStaged<int8_t, CIN, 32>(a, stream);

@@ -984,7 +984,12 @@ struct MMPlugin final : d3d_plugin {
     a.in = inputs[0];
     a.inNarrow = inputs[0];
     a.cinNarrow = cin;
-    if (dev->cinMfma > cin && (dtype == D3D_INT8 || ((reinterpret_cast<uintptr_t>(outputs[0]) & 15) == 0 &&
+    a.staged = stagedOverride();
+    if (dev->cinMfma > cin && a.staged == 0 && convReadsNarrowRows(dtype, kernelVol, cin, cout) &&
+        (reinterpret_cast<uintptr_t>(inputs[0]) & 15) == 0) {
+      a.cin = dev->cinMfma;       // the kernel reads the rows as they are and multiplies zeros for the rest
+      a.rowChannels = cin;
+    } else if (dev->cinMfma > cin && (dtype == D3D_INT8 || ((reinterpret_cast<uintptr_t>(outputs[0]) & 15) == 0 &&
                                                      debugEnv("D3D_CONV_NO_PAD") == nullptr))) {  // narrow layer: widen the rows, then MFMA
       if (!widened) widened = std::make_shared<DeviceBuffer>();
       const int es = dtypeBytes(dtype);
@@ -1012,7 +1017,6 @@ struct MMPlugin final : d3d_plugin {
     a.zeros = zeros;
     if (const char* e = debugEnv("D3D_CONV_PIPE")) a.pipe = e[0] == '0' ? -1 : 0;
     a.tileRows = tileRowsOverride();
-    a.staged = stagedOverride();
     return launchConv(a, stream);
   }
 };
