@@ -406,7 +406,11 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
 // (a stage row holding the neighbours under two taps side by side, the step of a 64-channel layer) measured slower
 // on both 32-channel layers in every tile shape tried (32 -> 32: 44-58 us against 37.5; 32 -> 64: 45-57 against
 // 36): the stage doubles, one workgroup fits a CU instead of two, and the layer needs the wavefronts more than
-// the longer steps.  Layers with few
+// the longer steps.  Smaller tiles for the sake of balance do not pay either: 351 000 rows are 686 tiles of 512 rows
+// on 512 workgroup slots (the busiest workgroup takes two), yet 384-row tiles (busiest: 768 rows) run the layer in
+// 43 us and 256-row tiles in 49 - a step costs about the same whatever its rows, because a CU's 16 wavefronts
+// move about 168 KB through LDS per step (gathered rows in and out, weight fragments) at 128 bytes per clock.
+// Layers with few
 // rows (the 128-channel stages: 47 000 rows are 186 tiles of 256 rows for 256 CUs) pick the workgroup shape by
 // tile count: the time of a layer that fits one round is that of ONE tile, so 248 tiles of 192 rows beat 186 of
 // 256 (48 us against 55), and there four wavefronts of 48 rows - one per SIMD, three 16-row groups each - beat
