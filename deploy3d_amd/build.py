@@ -21,13 +21,14 @@ ENGINE_LIB = os.path.join(LIBS, "libdeploy3d_amd.so")
 SYNTH_LIB = os.path.join(LIBS, "libd3d_synth.so")
 
 ENGINE_SOURCES = ["rulebook.hip", "conv.hip", "conv_half.hip", "conv_bf16.hip", "conv_int8.hip", "conv_pipe_half.hip",
-                  "conv_pipe_bf16.hip", "densify.hip", "voxelize.hip", "scratch.hip", "plugin.cpp", "schedule.cpp"]
+                  "conv_pipe_bf16.hip", "conv_pipe_int8.hip", "densify.hip", "voxelize.hip", "scratch.hip", "plugin.cpp", "schedule.cpp"]
 ENGINE_HEADERS = ["common.h", "conv_kernels.h", "conv_pipe.h", os.path.join(ROOT, "include", "d3d_spconv.h")]
 # per-source extra flags
 EXTRA_FLAGS = {
     # keeps the MFMA accumulators of the pipelined kernel in VGPRs (see the header of the two files)
     "conv_pipe_half.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "conv_pipe_bf16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "conv_pipe_int8.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 PEAKS_BIN = os.path.join(LIBS, "d3d_peaks")
 

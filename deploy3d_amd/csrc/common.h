@@ -176,6 +176,7 @@ int32_t launchMfmaInt8(const ConvArgs& a, hipStream_t stream);
 // The software-pipelined kernel (conv_pipe.h): 32 / 64 / 128 channels, kernel volumes up to 64.
 int32_t launchPipeHalf(const ConvArgs& a, hipStream_t stream);
 int32_t launchPipeBf16(const ConvArgs& a, hipStream_t stream);
+int32_t launchPipeInt8(const ConvArgs& a, hipStream_t stream);
 
 // True if the MFMA kernel family covers (dtype, cin, cout); otherwise the
 // narrow-channel kernel runs.

@@ -350,7 +350,9 @@ int32_t launchConv(const ConvArgs& a, hipStream_t stream) {
                "tensors and requantize scales");
       return D3D_ERR_UNSUPPORTED;
     }
-    rc = launchMfmaInt8(a, stream);
+    rc = D3D_ERR_UNSUPPORTED;
+    if (a.pipe >= 0 && a.staged == 0 && a.tileRows == 0 && a.rowChannels == 0) rc = launchPipeInt8(a, stream);
+    if (rc == D3D_ERR_UNSUPPORTED) rc = launchMfmaInt8(a, stream);
     if (rc == D3D_ERR_UNSUPPORTED) setError("conv: int8 layer does not fit the staged kernel (kernel volume %d)", a.kVol);
   } else if (convUsesMfma(a.dtype, a.cin, a.cout) && aligned && a.weightsMfma && a.zeros) {
     rc = D3D_ERR_UNSUPPORTED;

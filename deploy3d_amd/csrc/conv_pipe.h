@@ -1,4 +1,5 @@
-// Software-pipelined MFMA convolution for gfx950 (fp16 / bf16 storage, fp32 accumulation).
+// Software-pipelined MFMA convolution for gfx950 (fp16 / bf16 storage with fp32 accumulation; int8 storage with
+// int32 accumulation and a requantizing store, for rows of 64 or 128 bytes).
 //
 // Same mathematics and data layouts as convStaged (conv_kernels.h): output-stationary tiles, rows of a tap
 // gathered through the neighbour table into an XOR-swizzled LDS stage, weights in fragment-major order streamed
@@ -40,12 +41,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRawBuffer(const void* p, u
 template <class T, int CIN, int COUT, int MT, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES)
 convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf, const float* __restrict__ bias,
-         const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror,
+         const float* __restrict__ requantM, const int32_t* __restrict__ nbr, int64_t nbrPitch, int tapMirror,
          const unsigned long long* __restrict__ tileMasks, int kVol, int64_t inRows, int64_t outRows, int relu,
          int tileBlocks, int xcdShift, const int32_t* __restrict__ numActOut) {
   constexpr int THREADS = 64 * WAVES;
   constexpr int ES = static_cast<int>(sizeof(T));
-  constexpr int CS = CIN > 64 ? 64 : CIN;                      // input channels per step; a tap takes KS steps
+  constexpr int CS = CIN * ES > 128 ? 128 / ES : CIN;          // input channels per step (at most 128 bytes of a row); a tap takes KS steps
   constexpr int KS = CIN / CS;
   constexpr int CH = CS * ES / 16;                             // 16-byte chunks of a row staged per step
   constexpr int RPI = 64 / CH;                                 // rows one gather instruction covers
@@ -53,7 +54,7 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
   constexpr int GL = WM / RPI;                                 // gather instructions per step
   constexpr int GPM = 16 / RPI;                                // gathers that cover the 16 rows of one row group
   constexpr int NT = COUT / 16;
-  constexpr int KK = CS / 32;                                  // MFMA K = 32
+  constexpr int KK = CS * ES / 64;                             // MFMAs along K per step: 64 bytes of a row each
   constexpr int NQ = KK * NT;                                  // MFMAs per row group and step
   constexpr int WCH = CS * COUT * ES / 16;                     // 16-byte chunks of one step's weights
   constexpr int WL = (WCH + THREADS - 1) / THREADS;            // weight loads per wavefront and step
@@ -63,7 +64,7 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
   constexpr int SLOTS = WM * CH;                               // 16-byte slots of one stage
   constexpr int PER = TM / 64;                                 // tile masks per workgroup tile
   constexpr int ROWSHIFT = CIN * ES == 64 ? 6 : (CIN * ES == 128 ? 7 : 8);
-  static_assert(ES == 2 && (CS == 32 || CS == 64) && CIN % CS == 0 && WM % RPI == 0 && TM % 64 == 0, "shape");
+  static_assert((ES == 2 || ES == 1) && (CS * ES == 64 || CS * ES == 128) && CIN % CS == 0 && WM % RPI == 0 && TM % 64 == 0, "shape");
   static_assert((1 << ROWSHIFT) == CIN * ES && WCH % 64 == 0 && MT >= 2 && MT * NT * 4 <= 128, "shape");
   static_assert(WM < 64 || WM % 64 == 0, "an index load covers 64 rows: a wavefront tile is below 64 rows or whole multiples");
   using F = u32x4;
@@ -222,6 +223,34 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
       // channels this lane stores after the swaps: tile n for even 16-lane rows, tile n+1 for odd ones; the
       // first or second half of the tile's 16 channels by lane row / 2
       const int outCol = (n + (kgrp & 1)) * 16 + (kgrp >> 1) * 8;
+      if constexpr (ES == 1) {
+        // int8: q = clamp(rint(float(acc) * m[c] + bq[c])), lower bound 0 with the fused ReLU; a lane's 4 channels
+        // are one dword, and one swap hands every lane 8 consecutive channels
+        const float4v m0 = *reinterpret_cast<const float4v*>(requantM + col0);
+        const float4v m1 = *reinterpret_cast<const float4v*>(requantM + col1);
+        const float lo = relu ? 0.f : -128.f;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          uint32_t a = 0, c = 0;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            float t0 = static_cast<float>(acc[m][n][j]) * m0[j];
+            float t1 = static_cast<float>(acc[m][n + 1][j]) * m1[j];
+            t0 = t0 + b0[j];
+            t1 = t1 + b1[j];
+            const float q0 = __builtin_fminf(127.f, __builtin_fmaxf(lo, __builtin_rintf(t0)));
+            const float q1 = __builtin_fminf(127.f, __builtin_fmaxf(lo, __builtin_rintf(t1)));
+            a |= (static_cast<uint32_t>(static_cast<int>(q0)) & 0xFFu) << (8 * j);
+            c |= (static_cast<uint32_t>(static_cast<int>(q1)) & 0xFFu) << (8 * j);
+          }
+          acc[m][n] = Acc{0, 0, 0, 0};
+          acc[m][n + 1] = Acc{0, 0, 0, 0};
+          const auto sw = __builtin_amdgcn_permlane16_swap(a, c, false, false);
+          const u32x2 line = {sw[0], sw[1]};
+          const int64_t row = row0 + m * 16 + r16;
+          if (row < outRows) *reinterpret_cast<u32x2*>(out + static_cast<size_t>(row) * COUT + outCol) = line;
+        }
+      } else {
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         float v0[4], v1[4];
@@ -246,6 +275,7 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
         const u32x4 line = {s0[0], s1[0], s0[1], s1[1]};
         const int64_t row = row0 + m * 16 + r16;
         if (row < outRows) *reinterpret_cast<u32x4*>(out + static_cast<size_t>(row) * COUT + outCol) = line;
+      }
       }
     }
   };
@@ -365,7 +395,7 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
 
 template <class T, int CIN, int COUT, int MT, int WAVES>
 int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
-  constexpr int CS = CIN > 64 ? 64 : CIN;
+  constexpr int CS = CIN * static_cast<int>(sizeof(T)) > 128 ? 128 / static_cast<int>(sizeof(T)) : CIN;
   constexpr int WM = 16 * MT, TM = WM * WAVES;
   constexpr int WCH = CS * COUT * static_cast<int>(sizeof(T)) / 16;
   const size_t lds = static_cast<size_t>(3) * WCH * 16 + static_cast<size_t>(WAVES) * 2 * WM * (CS * sizeof(T)) +
@@ -390,8 +420,8 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
   if (blocks > chip.cus / nXcd * nXcd * perCu) blocks = chip.cus / nXcd * nXcd * perCu;
   hipLaunchKernelGGL((convPipe<T, CIN, COUT, MT, WAVES>), dim3(static_cast<unsigned>(blocks)), dim3(64 * WAVES),
                      lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
-                     static_cast<const T*>(a.weightsMfma), a.bias, a.nbr, pitch, a.tapMirror, a.tileMasks, a.kVol,
-                     a.inRows, a.outRows, a.relu, tiles, chip.xcdShift, a.numActOut);
+                     static_cast<const T*>(a.weightsMfma), a.bias, a.requantM, a.nbr, pitch, a.tapMirror, a.tileMasks,
+                     a.kVol, a.inRows, a.outRows, a.relu, tiles, chip.xcdShift, a.numActOut);
   return D3D_OK;
 }
 
@@ -417,7 +447,10 @@ int32_t launchPipeCfg(const ConvArgs& a, hipStream_t stream) {
 // six of 32 rows (45 us against 48).
 template <class T, int CIN, int COUT>
 int32_t launchPipeShape(const ConvArgs& a, hipStream_t stream) {
-  if constexpr (CIN == 64 && COUT == 64) {
+  // shapes go by the bytes of an input row (the stage) and by the output channels (the accumulators): an int8 layer
+  // takes the shape of the two-byte layer with half its input channels
+  constexpr int RB = CIN * static_cast<int>(sizeof(T));
+  if constexpr (RB == 128 && COUT == 64) {
     return launchPipeCfg<T, CIN, COUT, 4, 8>(a, stream);
   } else if constexpr (COUT >= 128) {
     // 8, 6 or 4 wavefronts of 32 rows: the workgroup size whose tiles load the busiest CU least (rounds of tiles
@@ -448,7 +481,7 @@ int32_t launchPipeShape(const ConvArgs& a, hipStream_t stream) {
     if (best == 2) return launchPipeCfg<T, CIN, COUT, 2, 4>(a, stream);
     if (best == 3) return launchPipeCfg<T, CIN, COUT, 3, 4>(a, stream);
     return launchPipeCfg<T, CIN, COUT, 2, 8>(a, stream);
-  } else if constexpr (CIN == 32 && COUT == 32) {
+  } else if constexpr (RB == 64 && COUT == 32) {
     return launchPipeCfg<T, CIN, COUT, 4, 8>(a, stream);
   } else {
     return launchPipeCfg<T, CIN, COUT, 4, 4>(a, stream);
@@ -459,9 +492,11 @@ template <class T>
 int32_t launchPipe(const ConvArgs& a, hipStream_t stream) {
 #define D3D_PIPE_CASE(CI, CO) \
   if (a.cin == CI && a.cout == CO) return launchPipeShape<T, CI, CO>(a, stream);
-  D3D_PIPE_CASE(32, 32)
-  D3D_PIPE_CASE(32, 64)
-  D3D_PIPE_CASE(32, 128)
+  if constexpr (sizeof(T) == 2) {  // rows of 64 bytes at least
+    D3D_PIPE_CASE(32, 32)
+    D3D_PIPE_CASE(32, 64)
+    D3D_PIPE_CASE(32, 128)
+  }
   D3D_PIPE_CASE(64, 32)
   D3D_PIPE_CASE(64, 64)
   D3D_PIPE_CASE(64, 128)

@@ -64,6 +64,28 @@ def test_int8_staged_configurations(engine, monkeypatch, cfg):
     run_int8(3001, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), 128, 32, True, False)
 
 
+@pytest.mark.parametrize("shape", ["32,8", "32,6", "32,4", "48,4"])
+@pytest.mark.parametrize("cin,cout", [(64, 128), (128, 128)])
+def test_int8_pipelined_tile_shapes(engine, monkeypatch, shape, cin, cout):
+    """Layers with rows of 64 bytes and more run the software-pipelined kernel; for 128 output channels it chooses
+    among four workgroup shapes by row count.  Each forced on a SubM layer with spare capacity and a strided one, and
+    once on a layer with more tiles than workgroups, where the pipeline runs across tiles."""
+    monkeypatch.setenv("D3D_CONV_PIPE_SHAPE", shape)
+    run_int8(9001, (12, 48, 40), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, True, True)
+    if cin == 64:
+        run_int8(5000, (12, 48, 40), (3, 3, 3), (2, 2, 2), (1, 1, 1), cin, cout, False, False)
+        run_int8(70000, (16, 200, 200), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, True, True)
+
+
+@pytest.mark.parametrize("cin,cout", [(64, 32), (64, 64), (128, 64), (128, 128)])
+def test_int8_pipelined_and_barrier_per_tap_kernels_agree_with_the_oracle(engine, monkeypatch, cin, cout):
+    """The same layer on the pipelined kernel (the default from 64 input channels up), across several tiles per
+    workgroup, and with the pipelined kernel switched off, which leaves the barrier-per-tap kernel."""
+    run_int8(40000, (16, 120, 120), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, True, True)
+    monkeypatch.setenv("D3D_CONV_PIPE", "0")
+    run_int8(3001, (10, 36, 30), (3, 3, 3), (1, 1, 1), (1, 1, 1), cin, cout, True, False)
+
+
 def test_int8_unsupported_channels_report_status(engine):
     from deploy3d_amd import EngineError
     with pytest.raises(EngineError) as e:
