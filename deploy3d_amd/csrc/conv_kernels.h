@@ -1123,7 +1123,9 @@ int32_t launchInt8Cout(const ConvArgs& a, hipStream_t stream) {
   return D3D_ERR_UNSUPPORTED;
 }
 
-inline int32_t launchInt8(const ConvArgs& a, hipStream_t stream) {
+// (a template so that only the translation unit that calls it instantiates the int8 kernels)
+template <class T = int8_t>
+int32_t launchInt8(const ConvArgs& a, hipStream_t stream) {
   switch (a.cin) {
     case 32: return launchInt8Cout<32>(a, stream);
     case 64: return launchInt8Cout<64>(a, stream);

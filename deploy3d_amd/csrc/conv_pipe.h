@@ -225,31 +225,38 @@ convPipe(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
       const int outCol = (n + (kgrp & 1)) * 16 + (kgrp >> 1) * 8;
       if constexpr (ES == 1) {
         // int8: q = clamp(rint(float(acc) * m[c] + bq[c])), lower bound 0 with the fused ReLU; a lane's 4 channels
-        // are one dword, and one swap hands every lane 8 consecutive channels
-        const float4v m0 = *reinterpret_cast<const float4v*>(requantM + col0);
-        const float4v m1 = *reinterpret_cast<const float4v*>(requantM + col1);
+        // are one dword, and one swap hands every lane 8 consecutive channels.  One channel tile at a time, so that
+        // only one set of scales is live beside the accumulators.
         const float lo = relu ? 0.f : -128.f;
+        uint32_t packed[2][MT];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int col = h ? col1 : col0;
+          const float4v mq = *reinterpret_cast<const float4v*>(requantM + col);
+          const float4v bq = h ? b1 : b0;
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              float t = static_cast<float>(acc[m][n + h][j]) * mq[j];
+              t = t + bq[j];
+              const float q = __builtin_fminf(127.f, __builtin_fmaxf(lo, __builtin_rintf(t)));
+              w |= (static_cast<uint32_t>(static_cast<int>(q)) & 0xFFu) << (8 * j);
+            }
+            packed[h][m] = w;
+            acc[m][n + h] = Acc{0, 0, 0, 0};
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-          uint32_t a = 0, c = 0;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            float t0 = static_cast<float>(acc[m][n][j]) * m0[j];
-            float t1 = static_cast<float>(acc[m][n + 1][j]) * m1[j];
-            t0 = t0 + b0[j];
-            t1 = t1 + b1[j];
-            const float q0 = __builtin_fminf(127.f, __builtin_fmaxf(lo, __builtin_rintf(t0)));
-            const float q1 = __builtin_fminf(127.f, __builtin_fmaxf(lo, __builtin_rintf(t1)));
-            a |= (static_cast<uint32_t>(static_cast<int>(q0)) & 0xFFu) << (8 * j);
-            c |= (static_cast<uint32_t>(static_cast<int>(q1)) & 0xFFu) << (8 * j);
-          }
-          acc[m][n] = Acc{0, 0, 0, 0};
-          acc[m][n + 1] = Acc{0, 0, 0, 0};
-          const auto sw = __builtin_amdgcn_permlane16_swap(a, c, false, false);
+          const auto sw = __builtin_amdgcn_permlane16_swap(packed[0][m], packed[1][m], false, false);
           const u32x2 line = {sw[0], sw[1]};
           const int64_t row = row0 + m * 16 + r16;
           if (row < outRows) *reinterpret_cast<u32x2*>(out + static_cast<size_t>(row) * COUT + outCol) = line;
         }
+        __builtin_amdgcn_sched_barrier(0);
       } else {
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
@@ -459,28 +466,41 @@ int32_t launchPipeShape(const ConvArgs& a, hipStream_t stream) {
     // others (conv4_x: 45 us against 48); over several rounds the eight-wavefront shapes hide their waits better
     // (a 64 -> 128 layer of 10 rounds: 105 us with 8 x 32 rows, 138 us with 4 x 48).
     static const int kCand[4][2] = {{32, 8}, {32, 6}, {32, 4}, {48, 4}};
-    int best = 0;
+    // int8 128 -> 128: the wider workgroups (two wavefronts per SIMD, 256 registers each) spill - 84-97 us against
+    // 33-44 on a 47 000-row layer - so only the four-wavefront shapes are candidates, the larger tile winning ties
+    constexpr bool FOUR_ONLY = sizeof(T) == 1 && CIN == 128;
+    int best = FOUR_ONLY ? 3 : 0;
     int64_t bestCost = 0;
-    for (int c = 0; c < 3; ++c) {
+    const int64_t cus = chipLayout().cus;
+    auto costOf = [&](int c) {
       const int64_t tm = kCand[c][0] * kCand[c][1], tiles = (a.outRows + tm - 1) / tm;
-      const int64_t cus = chipLayout().cus;
-      const int64_t cost = (tiles + cus - 1) / cus * tm;  // rows the busiest CU multiplies
-      if (c == 0 || cost < bestCost) {
-        best = c;
-        bestCost = cost;
+      return (tiles + cus - 1) / cus * tm;              // rows the busiest CU multiplies
+    };
+    if (FOUR_ONLY) {
+      if (costOf(2) < costOf(3)) best = 2;
+    } else {
+      for (int c = 0; c < 3; ++c) {
+        const int64_t cost = costOf(c);
+        if (c == 0 || cost < bestCost) {
+          best = c;
+          bestCost = cost;
+        }
       }
+      if (best == 1 && (a.outRows + 191) / 192 <= cus) best = 3;
     }
-    if (best == 1 && (a.outRows + 191) / 192 <= chipLayout().cus) best = 3;
     if (const char* force = debugEnv("D3D_CONV_PIPE_SHAPE")) {  // "rows,wavefronts" of one candidate (tests)
-      for (int c = 0; c < 4; ++c)
+      for (int c = FOUR_ONLY ? 2 : 0; c < 4; ++c)
         if (std::atoi(force) == kCand[c][0] && std::strchr(force, ',') &&
             std::atoi(std::strchr(force, ',') + 1) == kCand[c][1])
           best = c;
     }
-    if (best == 1) return launchPipeCfg<T, CIN, COUT, 2, 6>(a, stream);
     if (best == 2) return launchPipeCfg<T, CIN, COUT, 2, 4>(a, stream);
     if (best == 3) return launchPipeCfg<T, CIN, COUT, 3, 4>(a, stream);
-    return launchPipeCfg<T, CIN, COUT, 2, 8>(a, stream);
+    if constexpr (!FOUR_ONLY) {
+      if (best == 1) return launchPipeCfg<T, CIN, COUT, 2, 6>(a, stream);
+      return launchPipeCfg<T, CIN, COUT, 2, 8>(a, stream);
+    }
+    return D3D_ERR_UNSUPPORTED;
   } else if constexpr (RB == 64 && COUT == 32) {
     return launchPipeCfg<T, CIN, COUT, 4, 8>(a, stream);
   } else {
