@@ -315,13 +315,16 @@ convMfma(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf
 // its wavefronts walks, on its own, over groups of 16 output rows (group index strided by the number of
 // wavefronts in the grid), with a private slice of the neighbour table, its own list of the taps that occur
 // in the group, and no barrier after the weight load.  CROW < CIN: the rows of `in` store CROW channels only and
-// the lanes that would read the others multiply zeros (their weights are zero rows as well).
+// the lanes that would read the others multiply zeros (their weights are zero rows as well); CROW < 0: the rows
+// store `rowCh` channels, any number below CIN, and are read element by element (a 5-channel input: no widened
+// copy, and the few bytes of such rows do not need vector loads).
 template <class T, int CIN, int COUT, int WAVES, int CROW = CIN>
 __global__ void __launch_bounds__(64 * WAVES)
 convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restrict__ wf,
                  const float* __restrict__ bias, const float* __restrict__ requantM, const int32_t* __restrict__ nbr,
                  int64_t nbrPitch, int tapMirror, const T* __restrict__ zeros, int kVol, int64_t inRows,
-                 int64_t outRows, int relu, int groups, int xcdShift, const int32_t* __restrict__ numActOut) {
+                 int64_t outRows, int relu, int groups, int xcdShift, const int32_t* __restrict__ numActOut,
+                 int rowCh) {
   constexpr int THREADS = 64 * WAVES;
   constexpr int MT = 1;
   constexpr int NT = COUT / 16;
@@ -334,7 +337,7 @@ convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restr
   constexpr int WCHUNKS = CIN * COUT * ES / 16;
   using F = typename std::conditional<WIDE, u32x4, u32x2>::type;
   using Acc = typename Mfma<T>::Acc;
-  static_assert(CIN % KSTEP == 0 && (CROW == CIN || (KK == 1 && CROW % KG == 0)), "whole MFMA steps");
+  static_assert(CIN % KSTEP == 0 && (CROW == CIN || (KK == 1 && !WIDE && (CROW < 0 || CROW % KG == 0))), "whole MFMA steps");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   F* wLds = reinterpret_cast<F*>(smem);                                              // [kVol][WFRAGS]
@@ -353,10 +356,20 @@ convMfmaResident(const T* __restrict__ in, T* __restrict__ out, const T* __restr
 
   auto gatherRows = [&](int tap, F (&dst)[MT][KK]) __attribute__((always_inline)) {
     const int32_t src = tap < 0 ? -1 : nb[tap * 16 + r16];
-    const T* rowPtr = (src < 0 || kgrp * KG >= CROW ? zeros : in + static_cast<size_t>(src) * CROW + kgrp * KG);
-    if constexpr (CROW == CIN) rowPtr = (src < 0 ? zeros : in + static_cast<size_t>(src) * CIN) + kgrp * KG;
+    if constexpr (CROW < 0) {
+      T v[KG];
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) dst[0][kk] = *reinterpret_cast<const F*>(rowPtr + kk * KSTEP);
+      for (int j = 0; j < KG; ++j) {
+        const int ch = kgrp * KG + j;
+        v[j] = (src >= 0 && ch < rowCh) ? in[static_cast<size_t>(src) * rowCh + ch] : static_cast<T>(0);
+      }
+      dst[0][0] = __builtin_bit_cast(F, v);
+    } else {
+      const T* rowPtr = (src < 0 || kgrp * KG >= CROW ? zeros : in + static_cast<size_t>(src) * CROW + kgrp * KG);
+      if constexpr (CROW == CIN) rowPtr = (src < 0 ? zeros : in + static_cast<size_t>(src) * CIN) + kgrp * KG;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) dst[0][kk] = *reinterpret_cast<const F*>(rowPtr + kk * KSTEP);
+    }
   };
 
   // Workgroups are dealt to the XCDs round-robin; XCD x takes the x-th contiguous part of the row groups,
@@ -962,7 +975,7 @@ int32_t launchMfmaResident(const ConvArgs& a, hipStream_t stream) {
                      lds, stream, static_cast<const T*>(a.in), static_cast<T*>(a.out),
                      static_cast<const T*>(a.weightsMfma), a.bias, a.requantM, a.nbr,
                      a.nbrPitch > 0 ? a.nbrPitch : a.outRows, a.tapMirror, static_cast<const T*>(a.zeros), a.kVol,
-                     a.inRows, a.outRows, a.relu, groups, chip.xcdShift, a.numActOut);
+                     a.inRows, a.outRows, a.relu, groups, chip.xcdShift, a.numActOut, a.rowChannels);
   return D3D_OK;
 }
 
@@ -1021,19 +1034,30 @@ int32_t launchStaged(const ConvArgs& a, hipStream_t stream) {
   return D3D_ERR_UNSUPPORTED;
 }
 
+// Does the resident-weight kernel take the layer: every tap's weights and 16 wavefronts' table slices in LDS,
+// two workgroups per CU.
+inline bool residentFits(int kVol, int cin, int cout, size_t elemBytes) {
+  const size_t allTaps = static_cast<size_t>(kVol) * cin * cout * elemBytes;
+  return allTaps <= 56 * 1024 && kVol <= 128 && allTaps + static_cast<size_t>(16) * kVol * 16 * 4 <= kLdsLimit;
+}
+
 // Small layers keep every tap's weights in LDS (convMfmaResident).  Large layers stream one tap's weights at a
 // time through LDS for 8 (or 4) wavefronts; more rows per wavefront (MT) amortise that stream.
 template <class T, int CIN, int COUT>
 int32_t launchMfmaOne(const ConvArgs& a, hipStream_t stream) {
+  if (a.rowChannels > 0 && a.rowChannels < CIN) {  // narrow rows read as stored: the resident kernel only
+    if constexpr (CIN == 16 && (COUT == 16 || COUT == 32)) {
+      if (residentFits(a.kVol, CIN, COUT, sizeof(T))) return launchMfmaResident<T, CIN, COUT, -1>(a, stream);
+    }
+    return D3D_ERR_UNSUPPORTED;
+  }
   if constexpr (CIN * COUT >= 512) {
     if (a.staged >= 0) {
       const int32_t rc = launchStaged<T, CIN, COUT>(a, stream);
       if (rc != D3D_ERR_UNSUPPORTED) return rc;
     }
   }
-  const size_t allTaps = static_cast<size_t>(a.kVol) * CIN * COUT * sizeof(T);
-  if (allTaps <= 56 * 1024 && a.kVol <= 128 && allTaps + static_cast<size_t>(16) * a.kVol * 16 * 4 <= kLdsLimit)
-    return launchMfmaResident<T, CIN, COUT>(a, stream);
+  if (residentFits(a.kVol, CIN, COUT, sizeof(T))) return launchMfmaResident<T, CIN, COUT>(a, stream);
   // rows per workgroup = 16 * MT * WAVES
   int mt = 2;
   int waves = 8;
@@ -1087,10 +1111,7 @@ int32_t launchMfma(const ConvArgs& a, hipStream_t stream) {
 
 // Weights of every tap resident in LDS (register gathers, no barriers): what the 32-channel int8 layers of few
 // output channels run, like the 16-channel layers in two-byte types - their rows are as many bytes.
-inline bool int8ResidentFits(int kVol, int cin, int cout) {
-  const size_t allTaps = static_cast<size_t>(kVol) * cin * cout;
-  return allTaps <= 56 * 1024 && kVol <= 128 && allTaps + static_cast<size_t>(16) * kVol * 16 * 4 <= kLdsLimit;
-}
+inline bool int8ResidentFits(int kVol, int cin, int cout) { return residentFits(kVol, cin, cout, 1); }
 
 template <int CIN, int COUT, int CROW = CIN>
 int32_t launchInt8Resident(const ConvArgs& a, hipStream_t stream) {
@@ -1107,6 +1128,7 @@ int32_t launchInt8Cout(const ConvArgs& a, hipStream_t stream) {
       if (a.cout == 32) return launchInt8Resident<32, 32, 16>(a, stream);
       return D3D_ERR_UNSUPPORTED;
     }
+    if (a.rowChannels > 0) return D3D_ERR_UNSUPPORTED;
     if (a.staged == 0) {
       if (a.cout == 16) rc = launchInt8Resident<32, 16>(a, stream);
       if (a.cout == 32 && a.tileMasks == nullptr) rc = launchInt8Resident<32, 32>(a, stream);

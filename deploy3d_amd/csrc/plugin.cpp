@@ -986,7 +986,8 @@ struct MMPlugin final : d3d_plugin {
     a.cinNarrow = cin;
     a.staged = stagedOverride();
     if (dev->cinMfma > cin && a.staged == 0 && convReadsNarrowRows(dtype, kernelVol, cin, cout) &&
-        (reinterpret_cast<uintptr_t>(inputs[0]) & 15) == 0) {
+        ((reinterpret_cast<uintptr_t>(inputs[0]) | reinterpret_cast<uintptr_t>(outputs[0])) & 15) == 0 &&
+        (dtype == D3D_INT8 || debugEnv("D3D_CONV_NO_PAD") == nullptr) && tileRowsOverride() == 0) {
       a.cin = dev->cinMfma;       // the kernel reads the rows as they are and multiplies zeros for the rest
       a.rowChannels = cin;
     } else if (dev->cinMfma > cin && (dtype == D3D_INT8 || ((reinterpret_cast<uintptr_t>(outputs[0]) & 15) == 0 &&
