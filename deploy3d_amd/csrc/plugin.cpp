@@ -782,7 +782,8 @@ struct MMPlugin final : d3d_plugin {
     // Capacities are known here: reserve what enqueue would otherwise have to allocate on first use - the rows of a
     // narrow layer widened to the MFMA channel count, and the derived table of a node that has no link (or is an
     // inverse convolution, whose table is always derived).
-    if (in[0].nb_dims == 2 && in[0].dims[0] > 0 && dev->cinMfma > cin) {
+    if (in[0].nb_dims == 2 && in[0].dims[0] > 0 && dev->cinMfma > cin &&
+        !convReadsNarrowRows(dtype, kernelVol, cin, cout)) {
       if (!widened) widened = std::make_shared<DeviceBuffer>();
       const int32_t rc = widened->reserve(static_cast<size_t>(in[0].dims[0]) * dev->cinMfma * dtypeBytes(dtype));
       if (rc != D3D_OK) return rc;
@@ -930,6 +931,11 @@ struct MMPlugin final : d3d_plugin {
       return D3D_ERR_BAD_ARG;
     }
     if (dev->dtype != dtype) {  // a plugin enqueued without configurePlugin, or with another dtype
+      if (streamIsCapturing(stream)) {  // converting and uploading the weights allocates and synchronises
+        setError("SPConvMM: the node was not configured for this feature type before the capture (call "
+                 "d3d_configure, or enqueue it once, first)");
+        return D3D_ERR_UNSUPPORTED;
+      }
       int32_t rc = configure(inDesc, 1, nullptr, 0);
       if (rc != D3D_OK) return rc;
     }

@@ -381,3 +381,55 @@ def test_random_layers(engine):
         run_case(int(rng.integers(200, 2500)), (10, 30, 28), ksize, stride, padding, cin, cout, dtype, subm,
                  with_bias=bool(rng.integers(0, 2)), relu=bool(rng.integers(0, 2)), inverse=inverse, seed=100 + i,
                  cap_extra=int(rng.integers(0, 3)) * 37)
+
+
+def test_an_unprepared_node_is_refused_under_capture(engine):
+    """Under stream capture an enqueue neither allocates nor synchronises.  A node that was never configured (its
+    weights are not on the device, its derived table not reserved) reports UNSUPPORTED there; a node configured from
+    its descriptors captures without ever having been enqueued, and so does the first one after an eager enqueue;
+    replays give the eager result."""
+    from deploy3d_amd import EngineError
+    from deploy3d_amd.plugin import Plugin, TensorDesc
+    from deploy3d_amd.spconv_mm import mm_blob, run_mm
+    rng = np.random.default_rng(77)
+    grid, ksize = (10, 36, 30), (3, 3, 3)
+    coords = random_cloud(rng, 2000, grid, 1)
+    n = len(coords)
+    rb = gpu_rulebook(coords, n, grid, 1, ksize, (1, 1, 1), (1, 1, 1), (1, 1, 1), n, True)
+    w = round_to(rng.standard_normal((27, 32, 32)) / 30.0, "float16")
+    b = round_to(rng.standard_normal(32), "float16")
+    x = torch.from_numpy(round_to(rng.standard_normal((n, 32)), "float16")).to(device="cuda", dtype=torch.float16)
+    out = torch.empty((n, 32), dtype=torch.float16, device="cuda")
+    args = (x, rb["num_act_in"], rb["num_act_in"], rb["dev"][0], rb["dev"][1])
+    ref = oracle.conv(x.float().cpu().numpy(), w, b, rb["index"], rb["num_index"], n, acc="f64")
+
+    def captured(plugin):
+        graph, err = torch.cuda.CUDAGraph(), None
+        with torch.cuda.graph(graph):
+            try:
+                run_mm(plugin, *args, out=out)
+            except EngineError as e:
+                err = e
+        return graph, err
+
+    def replayed(graph):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        return out.clone()
+
+    fresh = Plugin("SPConvMM", mm_blob(ksize, 32, 32, n, True, False, w, b))
+    _, err = captured(fresh)
+    assert err is not None and err.status == -1 and "capture" in str(err)
+    configured = Plugin("SPConvMM", mm_blob(ksize, 32, 32, n, True, False, w, b))
+    in_descs = [TensorDesc.of_tensor(t) for t in args]
+    configured.configure(in_descs, configured.output_descs(in_descs))
+    graph, err = captured(configured)
+    assert err is None
+    check_close(replayed(graph).float().cpu().numpy(), ref, "float16")
+    eager = run_mm(fresh, *args, out=out).clone()      # one eager enqueue reserves everything
+    torch.cuda.synchronize()
+    check_close(eager.float().cpu().numpy(), ref, "float16")
+    graph, err = captured(fresh)
+    assert err is None
+    assert torch.equal(replayed(graph), eager)
