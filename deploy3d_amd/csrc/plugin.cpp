@@ -439,7 +439,44 @@ struct IdxPlugin final : d3d_plugin {
     if (!io || pos < 0 || pos >= nbIn + nbOut) return 0;
     return io[pos].format == D3D_LINEAR && io[pos].dtype == D3D_INT32;  // index_trt.cu:156-161
   }
-  int32_t configure(const d3d_tensor_desc*, int32_t, const d3d_tensor_desc*, int32_t) override { return D3D_OK; }
+  // The operator-owned pair of block maps (and their state words) for this grid and capacity: kept between passes
+  // for the SubM operators linked to this one's outputs, and - two maps in turn - so that a build needs no reset
+  // pass.  The two alternate cleanly only among builds on one grid size: another size takes a new, zeroed
+  // allocation.  `mayAllocate` false (a stream under capture): only says whether they are there.  Caller holds
+  // link->mutex.
+  bool mapsReady(const RbGeom& g, int64_t cap, bool mayAllocate) {
+    size_t recBytes = 0, chunkBytes = 0;
+    blockMapBytes(g, cap, &recBytes, &chunkBytes);
+    if (!recBytes) return false;
+    const size_t stateBytes = mapStateWords(chunkBytes) * 4;
+    auto have = [&]() {
+      return link->mapRecords.bytes >= 2 * recBytes && link->mapChunkBase.bytes >= chunkBytes &&
+             link->mapState.bytes >= stateBytes && link->mapStride * 16 == static_cast<int64_t>(recBytes);
+    };
+    if (!have() && mayAllocate) {
+      link->mapStride = 0;
+      if (link->mapRecords.reallocZeroed(2 * recBytes) == D3D_OK && link->mapChunkBase.reserve(chunkBytes) == D3D_OK &&
+          link->mapState.reallocZeroed(stateBytes) == D3D_OK) {
+        link->mapStride = static_cast<int64_t>(recBytes / 16);
+        link->mapDirty = false;
+      }
+    }
+    return have();
+  }
+  bool keepsItsMap() const { return (!subM && link->shareMap) || persistentIndex; }
+
+  // configurePlugin (index_trt.cu:153-159 does nothing): capacities and grid are known here, so the maps an
+  // operator keeps are reserved now and an enqueue - under capture or not - finds them.
+  int32_t configure(const d3d_tensor_desc* in, int32_t nbIn, const d3d_tensor_desc*, int32_t) override {
+    if (!in || nbIn < 3 || in[0].nb_dims != 2 || in[0].dims[1] != nd + 1 || in[2].nb_dims != nd + 2) return D3D_OK;
+    int32_t grid[kMaxSpatial + 1], inGrid[kMaxSpatial + 1];
+    outputGrid(in[2], grid);
+    inGrid[0] = in[2].dims[0];
+    for (int i = 0; i < nd; ++i) inGrid[1 + i] = in[2].dims[2 + i];
+    std::lock_guard<std::mutex> lock(link->mutex);
+    if (keepsItsMap()) (void)mapsReady(geometry(grid, inGrid), in[0].dims[0], true);
+    return D3D_OK;
+  }
 
   RbGeom geometry(const int32_t* outGrid /* [B, spatial...] */, const int32_t* inGrid = nullptr) const {
     RbGeom g{};
@@ -533,29 +570,12 @@ struct IdxPlugin final : d3d_plugin {
     // outputs, a SubM operator takes the map of the operator that wrote the coordinates it is handed
     std::shared_ptr<RulebookLink> source = subM ? coordSource : nullptr;
     std::unique_lock<std::mutex> sourceLock;
-    if (((!subM && link->shareMap) || persistentIndex) && !g_noAlloc) {
-      // The map is kept in memory of this operator: for the SubM operators linked to its outputs, and - two maps
-      // in turn - so that a build needs no reset pass.  Allocated (and zeroed) on first use, or when the grid
-      // grows; never while the stream is being captured.
-      size_t recBytes = 0, chunkBytes = 0;
-      blockMapBytes(g, cap, &recBytes, &chunkBytes);
+    if (keepsItsMap() && !g_noAlloc) {
+      // allocated (and zeroed) on first use unless configure did it, or when the grid grows; never while the stream
+      // is being captured
       hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
       (void)hipStreamIsCapturing(stream, &capturing);
-      const size_t stateBytes = mapStateWords(chunkBytes) * 4;
-      // the two maps alternate cleanly only among builds on one grid size: another size takes a new allocation
-      auto have = [&]() {
-        return link->mapRecords.bytes >= 2 * recBytes && link->mapChunkBase.bytes >= chunkBytes &&
-               link->mapState.bytes >= stateBytes && link->mapStride * 16 == static_cast<int64_t>(recBytes);
-      };
-      if (recBytes && !have() && capturing == hipStreamCaptureStatusNone) {
-        link->mapStride = 0;
-        if (link->mapRecords.reallocZeroed(2 * recBytes) == D3D_OK && link->mapChunkBase.reserve(chunkBytes) == D3D_OK &&
-            link->mapState.reallocZeroed(stateBytes) == D3D_OK) {
-          link->mapStride = static_cast<int64_t>(recBytes / 16);
-          link->mapDirty = false;
-        }
-      }
-      if (recBytes && have()) {
+      if (mapsReady(g, cap, capturing == hipStreamCaptureStatusNone)) {
         side.mapRecords = link->mapRecords.ptr;
         side.mapChunkBase = static_cast<uint32_t*>(link->mapChunkBase.ptr);
         side.mapState = static_cast<uint32_t*>(link->mapState.ptr);

@@ -91,6 +91,7 @@ class SparseConvLayer:
             # a SubM rulebook on the outputs of a strided one reuses that operator's occupancy map
             if self.spec["subm"] and self.extensions:
                 self.idx_plugin.link_coords(x.producer)
+            self.idx_plugin.configure(in_descs, out_descs)  # reserves the maps an operator keeps between passes
         st = self._idx_state
         self.idx_plugin.enqueue(st["in_descs"], st["out_descs"], [x.coors, x.num_act, None], st["outs"], st["ws"])
         outs = st["outs"]

@@ -293,6 +293,51 @@ def test_persistent_index_tensor(engine):
         plugin.close()
 
 
+def test_configured_operator_captures_without_an_eager_pass(engine):
+    """An operator that keeps its occupancy map between passes (persistent index tensor) reserves its two maps at
+    configure: captured in a graph without ever having been enqueued eagerly, every replay - the maps take turns
+    from replay to replay - on changing clouds gives the oracle's rulebook."""
+    import torch
+    from deploy3d_amd.plugin import OPT_PERSISTENT_INDEX, Plugin, TensorDesc
+    from deploy3d_amd.spconv_index import index_blob
+    grid, cap = (12, 40, 33), 4000
+    rng = np.random.default_rng(78)
+    for subm, stride in ((True, (1, 1, 1)), (False, (2, 2, 2))):
+        max_out = cap if subm else 8 * cap
+        args = ((3, 3, 3), stride, (1, 1, 1), (1, 1, 1))
+        plugin = Plugin("SPConvIdx3d", index_blob(*args, (0, 0, 0), max_out, subm, False))
+        plugin.set_option(OPT_PERSISTENT_INDEX, 1)
+        coors = torch.zeros((cap, 4), dtype=torch.int32, device="cuda")
+        num = torch.zeros(1, dtype=torch.int32, device="cuda")
+        in_descs = [TensorDesc.of_tensor(coors), TensorDesc.of_tensor(num), TensorDesc.of((1, 0) + grid, torch.int32)]
+        out_descs = plugin.output_descs(in_descs)
+        outs = [torch.empty(d.shape(), dtype=torch.int32, device="cuda") for d in out_descs]
+        ws = torch.empty(max(1, plugin.workspace_size(in_descs, out_descs)), dtype=torch.uint8, device="cuda")
+        plugin.configure(in_descs, out_descs)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            plugin.enqueue(in_descs, out_descs, [coors, num, None], outs, ws)
+        out_grid = (1,) + (grid if subm else tuple(out_descs[4].shape()[2:]))
+        for n in (3000, 700, 4000, 1500):
+            coords = random_cloud(rng, n, grid, 1)
+            coors.zero_()
+            coors[:n] = torch.from_numpy(coords).cuda()
+            num.fill_(n)
+            graph.replay()
+            torch.cuda.synchronize()
+            ref = oracle.rulebook(coors.cpu().numpy(), n, out_grid, *args, max_out, subm)
+            index, ni = outs[0].cpu().numpy(), int(outs[1].item())
+            assert ni == ref["num_index"]
+            if subm:
+                np.testing.assert_array_equal(index[:, :ni], ref["index"][:, :ni])
+            else:
+                c_ref, t_ref = oracle.canonical(ref["index"], ref["num_index"], ref["out_coors"], ref["num_act_out"])
+                c_got, t_got = oracle.canonical(index, ni, outs[2].cpu().numpy(), int(outs[3].item()))
+                np.testing.assert_array_equal(c_got, c_ref)
+                np.testing.assert_array_equal(t_got, t_ref)
+        plugin.close()
+
+
 def _random_geometry(rng):
     """A random but valid layer: 1 to 4 dims, kernel 1..5, stride 1..3, padding 0..2, dilation 1..2."""
     nd = int(rng.integers(1, 5))
