@@ -118,6 +118,16 @@ struct RbSide {
   bool mapDouble = false;               // out: the build alternated between the two maps (in, with useSharedMap:
                                         // the build that wrote the shared map did)
   bool mapDirty = false;                // a build with a reset pass has used these maps: keep the reset pass
+  // A strided build whose input rows are the outputs of another strided build (rows in rank order of that
+  // build's map, srcRows of them at capacity) may be handed that finished map of its INPUT grid: for the kernel
+  // shapes it knows (3x3x3 stride 2 padding 1; 3x1x1 stride (2,1,1) padding 0) it then derives the occupancy of
+  // every output brick from the input bricks underneath, inside the scan pass - no marking pass, no atomics.
+  const void* srcRecords = nullptr;
+  const uint32_t* srcChunkBase = nullptr;
+  uint32_t* srcState = nullptr;         // with srcDouble: the source's mapState (which of its two maps is finished)
+  int64_t srcStride = 0;
+  bool srcDouble = false;
+  bool sourceMapUsed = false;           // out
 };
 
 // 32-bit words of RbSide::mapState for a map of `chunkBaseBytes` bytes of chunk bases.

@@ -303,7 +303,7 @@ struct IdxPlugin final : d3d_plugin {
   bool persistentIndex = false;                  // D3D_OPT_PERSISTENT_INDEX
   bool indexUnused = false;                      // D3D_OPT_INDEX_UNUSED
   std::shared_ptr<RulebookLink> link = std::make_shared<RulebookLink>();  // by-products for linked convolutions
-  std::shared_ptr<RulebookLink> coordSource;     // SubM: record of the strided operator that writes inCoors
+  std::shared_ptr<RulebookLink> coordSource;     // record of the strided operator that writes inCoors (d3d_link_coords)
 
   int kVol() const {
     int v = 1;
@@ -568,7 +568,7 @@ struct IdxPlugin final : d3d_plugin {
     }
     // one block map per stage (d3d_link_coords): a strided operator keeps its map for the SubM operators on its
     // outputs, a SubM operator takes the map of the operator that wrote the coordinates it is handed
-    std::shared_ptr<RulebookLink> source = subM ? coordSource : nullptr;
+    std::shared_ptr<RulebookLink> source = coordSource;
     std::unique_lock<std::mutex> sourceLock;
     if (keepsItsMap() && !g_noAlloc) {
       // allocated (and zeroed) on first use unless configure did it, or when the grid grows; never while the stream
@@ -588,14 +588,21 @@ struct IdxPlugin final : d3d_plugin {
       sourceLock = std::unique_lock<std::mutex>(source->mutex);
       bool same = source->mapValid && source->mapCoors == inputs[0] && source->mapNumAct == inputs[1] &&
                   source->mapNd == nd && source->mapRows == cap;
-      for (int i = 0; same && i <= nd; ++i) same = source->mapGrid[i] == grid[i];
-      if (same) {
+      for (int i = 0; same && i <= nd; ++i) same = source->mapGrid[i] == inGrid[i];  // (SubM: the output grid too)
+      if (same && subM) {
         side.mapRecords = source->mapRecords.ptr;
         side.mapChunkBase = static_cast<uint32_t*>(source->mapChunkBase.ptr);
         side.mapState = static_cast<uint32_t*>(source->mapState.ptr);
         side.mapStride = source->mapStride;
         side.mapDouble = source->mapDouble;
         side.useSharedMap = true;
+      } else if (same) {
+        // a strided operator on another's outputs: that operator's map is the map of THIS one's input cells
+        side.srcRecords = source->mapRecords.ptr;
+        side.srcChunkBase = static_cast<const uint32_t*>(source->mapChunkBase.ptr);
+        side.srcState = static_cast<uint32_t*>(source->mapState.ptr);
+        side.srcStride = source->mapStride;
+        side.srcDouble = source->mapDouble;
       }
     }
     link->tableValid = link->masksValid = false;
@@ -1466,8 +1473,8 @@ int32_t d3d_link_rulebook(d3d_plugin* mm, d3d_plugin* idx) {
 int32_t d3d_link_coords(d3d_plugin* subm, d3d_plugin* producer) {
   D3D_GUARD_BEGIN
   auto* s = dynamic_cast<IdxPlugin*>(subm);
-  if (!s || !s->subM) {
-    setError("d3d_link_coords: the first handle must be a submanifold SPConvIdx{N}d");
+  if (!s) {
+    setError("d3d_link_coords: the first handle must be an SPConvIdx{N}d");
     return D3D_ERR_BAD_ARG;
   }
   if (!producer) {

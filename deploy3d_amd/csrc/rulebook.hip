@@ -1037,13 +1037,132 @@ __device__ __forceinline__ uint32_t pick(bool c, uint32_t a, uint32_t b) {
 
 constexpr uint32_t kScanGroup = 32;  // workgroups of the scan pass that share one first-level ticket
 
-// One pass over the records: every record gets the count of occupied cells before it INSIDE its chunk of 1024
-// records, every chunk its total; the workgroup that finishes last (a ticket counter, no waiting) turns the chunk
-// totals into exclusive chunk bases and writes numActOut = min(total, maxNumActOut) for strided convolutions.
-template <bool ORDERED>
-__global__ void __launch_bounds__(kRbThreads)
+// What a scan that derives its occupancy from the map of the input grid needs (bmScan<.., GATHER>).
+struct GatherArgs {
+  RecRef src;                      // finished map of the input grid (rows of the input = ranks in it)
+  const uint32_t* srcChunkBase;
+  BlockMap mo, mi;                 // bricks of the output grid / of the input grid
+  const int32_t* numActIn;
+  uint32_t inCap;                  // row capacity of the input: a live count below it rules truncation out
+  int shapeY, shapeX;              // output extents of the two in-brick dims
+  int padZ;                        // GATHER 1: padding of the level dim, 0 or 1
+};
+
+// Cells of an input-map record (bits, rank `first` of its lowest cell) that are rows of the input: cells ranked at
+// or past nLive were cut off when the build that wrote the map truncated its outputs.
+__device__ __forceinline__ unsigned long long cutToLive(unsigned long long bits, uint32_t first, uint32_t nLive) {
+  if (first >= nLive) return 0ull;
+  uint32_t n = static_cast<uint32_t>(__popcll(bits));
+  while (first + n > nLive) {  // at most one record of the map is cut inside
+    bits &= ~(1ull << (63 - __builtin_clzll(bits)));
+    --n;
+  }
+  return bits;
+}
+
+// bits 0, 2, .., 14 of x packed into bits 0..7
+__device__ __forceinline__ uint32_t evenBits(uint32_t x) {
+  x &= 0x5555u;
+  x = (x | (x >> 1)) & 0x3333u;
+  x = (x | (x >> 2)) & 0x0F0Fu;
+  x = (x | (x >> 4)) & 0x00FFu;
+  return x;
+}
+
+// Occupancy of output record `rec` (a brick of 1 x 8 x 8 cells) from the input map.
+//   GATHER 1: 3x3x3, stride 2, padding (pz, 1, 1) with pz 0 or 1: output (z, y, x) has a pair when any input cell of
+//             (2z-pz..2z-pz+2, 2y-1..2y+1, 2x-1..2x+1) is a row: 3 levels of 3 x 3 input bricks.
+//   GATHER 2: 3x1x1, stride (2,1,1), padding 0: input levels 2z..2z+2 of the same brick.
+template <int GATHER>
+__device__ __forceinline__ unsigned long long gatherOccupancy(const GatherArgs& ga, const BmRecord* __restrict__ src,
+                                                              uint32_t rec, uint32_t nLive, bool checkRanks) {
+  uint32_t q = rec;
+  const int obx = static_cast<int>(q % static_cast<uint32_t>(ga.mo.nb[3]));
+  q /= static_cast<uint32_t>(ga.mo.nb[3]);
+  const int oby = static_cast<int>(q % static_cast<uint32_t>(ga.mo.nb[2]));
+  q /= static_cast<uint32_t>(ga.mo.nb[2]);
+  const int oz = static_cast<int>(q % static_cast<uint32_t>(ga.mo.nb[1]));
+  const uint32_t batch = q / static_cast<uint32_t>(ga.mo.nb[1]);  // the leading spatial dim of a 3-D grid has extent 1
+  const int nz = ga.mi.nb[1], ny = ga.mi.nb[2], nx = ga.mi.nb[3];
+  constexpr int NA = GATHER == 1 ? 3 : 1;           // input bricks under the output brick per in-brick dim
+  constexpr int N = 3 * NA * NA;
+  // Every record underneath is requested before the first is looked at - the loads are independent - and only
+  // its occupancy bits are (8 bytes; 27 whole records would not fit the registers of a 1024-thread workgroup).
+  // A brick outside the grid reads record 0 and counts as empty.
+  auto recordAt = [&](int e, bool* inside) -> uint32_t {
+    const int dz = e / (NA * NA), a = (e / NA) % NA, c = e % NA;
+    const int iz = GATHER == 1 ? 2 * oz + dz - ga.padZ : 2 * oz + dz;
+    const int iby = GATHER == 1 ? 2 * oby + a - 1 : oby;
+    const int ibx = GATHER == 1 ? 2 * obx + c - 1 : obx;
+    *inside = iz >= 0 && iz < nz && iby >= 0 && iby < ny && ibx >= 0 && ibx < nx;
+    return *inside ? ((batch * static_cast<uint32_t>(nz) + static_cast<uint32_t>(iz)) * static_cast<uint32_t>(ny) +
+                      static_cast<uint32_t>(iby)) * static_cast<uint32_t>(nx) + static_cast<uint32_t>(ibx)
+                   : 0u;
+  };
+  uint2 got[N];
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    bool inside;
+    const uint32_t at = recordAt(e, &inside);
+    got[e] = *reinterpret_cast<const uint2*>(src + at);
+    if (!inside) got[e] = make_uint2(0u, 0u);
+  }
+  unsigned long long under[NA][NA];  // [brick row][brick column] of the input bricks, the three levels merged
+#pragma unroll
+  for (int a = 0; a < NA; ++a)
+#pragma unroll
+    for (int c = 0; c < NA; ++c) under[a][c] = 0ull;
+  if (!checkRanks) {  // grid-uniform
+#pragma unroll
+    for (int e = 0; e < N; ++e) under[(e / NA) % NA][e % NA] |= (static_cast<unsigned long long>(got[e].y) << 32) | got[e].x;
+  } else {
+#pragma unroll 1
+    for (int e = 0; e < N; ++e) {
+      bool inside;
+      const uint32_t at = recordAt(e, &inside);
+      if (!inside) continue;
+      const uint4 r = *reinterpret_cast<const uint4*>(src + at);
+      unsigned long long bits = (static_cast<unsigned long long>(r.y) << 32) | r.x;
+      if (bits) bits = cutToLive(bits, ga.srcChunkBase[at / kRbChunk] + r.z, nLive);
+      // (a loop that is not unrolled: the brick is chosen by arithmetic, not by a constant index)
+      const int a = (e / NA) % NA, c = e % NA;
+#pragma unroll
+      for (int aa = 0; aa < NA; ++aa)
+#pragma unroll
+        for (int cc = 0; cc < NA; ++cc)
+          if (aa == a && cc == c) under[aa][cc] |= bits;
+    }
+  }
+  if constexpr (GATHER == 2) {
+    return under[0][0];
+  } else {
+    // input row i of the 17 under the brick (i = 0: the last row of the brick row above) as 17 cells: bit 0 the
+    // last cell of the brick to the left, bits 1..16 the cells of the two bricks underneath
+    auto row17 = [&](int i) -> uint32_t {
+      const int a = i == 0 ? 0 : (i <= 8 ? 1 : 2);
+      const int sh = 8 * (i == 0 ? 7 : (i <= 8 ? i - 1 : i - 9));
+      const uint32_t l = static_cast<uint32_t>(under[a][0] >> sh) & 0xFFu, m = static_cast<uint32_t>(under[a][1] >> sh) & 0xFFu,
+                     r = static_cast<uint32_t>(under[a][2] >> sh) & 0xFFu;
+      return (l >> 7) | (m << 1) | (r << 9);
+    };
+    unsigned long long bits = 0ull;
+#pragma unroll
+    for (int oy = 0; oy < 8; ++oy) {
+      const uint32_t x = row17(2 * oy) | row17(2 * oy + 1) | row17(2 * oy + 2);
+      bits |= static_cast<unsigned long long>(evenBits(x | (x >> 1) | (x >> 2))) << (8 * oy);
+    }
+    return bits;
+  }
+}
+
+// GATHER != 0: the occupancy bits are not in the map yet (no marking pass ran) - they are derived here from the
+// map of the input grid (gatherOccupancy) and stored with the prefix.
+// That variant runs 1024 threads per workgroup: one thread per record of the chunk gathers (27 independent loads),
+// the bits pass through LDS, and the first 256 threads go on with the scan as always.
+template <bool ORDERED, int GATHER>
+__global__ void __launch_bounds__(GATHER ? kRbChunk : kRbThreads)
 bmScan(RecRef recRef, uint32_t nRecords, uint32_t* chunkBase, uint32_t nChunks, uint32_t* ticket,
-       uint32_t* groupTickets, int32_t* numActOut, int32_t maxNumActOut) {
+       uint32_t* groupTickets, int32_t* numActOut, int32_t maxNumActOut, GatherArgs ga) {
   __shared__ uint32_t scratch[kRbThreads / 64];
   __shared__ uint32_t isLast;
   const uint32_t epoch = recRef.epoch ? *recRef.epoch : 0u;
@@ -1057,9 +1176,37 @@ bmScan(RecRef recRef, uint32_t nRecords, uint32_t* chunkBase, uint32_t nChunks, 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t first = blockIdx.x * kRbChunk + wave * 256 + lane;
   uint32_t count[kRbItems];
+  unsigned long long gathered[GATHER ? kRbItems : 1];
+  if constexpr (GATHER != 0) {
+    __shared__ unsigned long long chunkBits[kRbChunk];
+    {
+      const BmRecord* __restrict__ src = ga.src.get();
+      const int32_t live = *ga.numActIn;
+      const uint32_t nLive = live < 0 ? 0u : (static_cast<uint32_t>(live) < ga.inCap ? static_cast<uint32_t>(live) : ga.inCap);
+      const bool checkRanks = nLive >= ga.inCap;  // fewer rows than the capacity: nothing was cut off
+      const uint32_t rec = blockIdx.x * kRbChunk + threadIdx.x;
+      unsigned long long bits = rec < nRecords ? gatherOccupancy<GATHER>(ga, src, rec, nLive, checkRanks) : 0ull;
+      if (bits) {  // cells of the brick past the edge of the output grid are no outputs
+        const int by = static_cast<int>((rec / static_cast<uint32_t>(ga.mo.nb[3])) % static_cast<uint32_t>(ga.mo.nb[2]));
+        const int bx = static_cast<int>(rec % static_cast<uint32_t>(ga.mo.nb[3]));
+        const int rows = ga.shapeY - 8 * by, cols = ga.shapeX - 8 * bx;
+        if (rows < 8) bits &= (1ull << (8 * rows)) - 1ull;
+        if (cols < 8) bits &= 0x0101010101010101ull * ((1ull << cols) - 1ull);
+      }
+      chunkBits[threadIdx.x] = bits;
+    }
+    __syncthreads();
+    if (threadIdx.x >= kRbThreads) return;  // (a wavefront that has ended no longer counts at a barrier)
+#pragma unroll
+    for (int j = 0; j < kRbItems; ++j) {
+      gathered[j] = chunkBits[wave * 256 + j * 64 + lane];
+      count[j] = static_cast<uint32_t>(__popcll(gathered[j]));
+    }
+  }
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
-    count[j] = first + j * 64 < nRecords ? static_cast<uint32_t>(__popcll(records[first + j * 64].bits)) : 0u;
+    if constexpr (GATHER == 0)
+      count[j] = first + j * 64 < nRecords ? static_cast<uint32_t>(__popcll(records[first + j * 64].bits)) : 0u;
     if (other && first + j * 64 < nRecords) other[first + j * 64].bits = 0ull;
   }
   uint32_t inclA = count[0] | (count[1] << 16), inclB = count[2] | (count[3] << 16);
@@ -1085,7 +1232,15 @@ bmScan(RecRef recRef, uint32_t nRecords, uint32_t* chunkBase, uint32_t nChunks, 
 #pragma unroll
   for (int j = 0; j < kRbItems; ++j) {
     // an empty record is never ranked: on sparse grids most are
-    if (count[j]) records[first + j * 64].prefix = rank + incl[j] - count[j];
+    if constexpr (GATHER != 0) {
+      if (count[j]) {
+        const unsigned long long bits = gathered[j];
+        *reinterpret_cast<uint4*>(records + first + j * 64) =
+            make_uint4(static_cast<uint32_t>(bits), static_cast<uint32_t>(bits >> 32), rank + incl[j] - count[j], 0u);
+      }
+    } else {
+      if (count[j]) records[first + j * 64].prefix = rank + incl[j] - count[j];
+    }
     rank += rowSum[j];
   }
   if (threadIdx.x == 0) {
@@ -1142,7 +1297,7 @@ bmScan(RecRef recRef, uint32_t nRecords, uint32_t* chunkBase, uint32_t nChunks, 
   // the finished one, the next build marks the other.
   if (recRef.epoch) {
     const uint32_t nGroups = (nChunks + kScanGroup - 1) / kScanGroup;
-    for (uint32_t q = threadIdx.x; q < nGroups; q += blockDim.x) groupTickets[q] = 0u;
+    for (uint32_t q = threadIdx.x; q < nGroups; q += kRbThreads) groupTickets[q] = 0u;
     if (threadIdx.x == 0) {
       *ticket = 0u;
       *recRef.epoch = epoch + 1u;
@@ -2069,8 +2224,39 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
                          resetFill, resetFillN, reinterpret_cast<uint32_t*>(cnt),
                          static_cast<int64_t>((w.totals - w.cnt) / 4 + totalsWords(g.kVol, w.nChunks)),
                          numIndex, masks, nMasks, fillState);
+    // A strided build on the outputs of another strided build, handed that build's finished map: the occupancy of
+    // its own map is derived from it inside the scan (bmScan<.., GATHER>), the marking pass and its atomics go.
+    int gather = 0;
+    GatherArgs ga{};
+    if (!subM && !g.transpose && near && side.srcRecords && side.srcChunkBase && g.nd == 3 && ksel != 0) {
+      const bool cube = ksel == 1 && g.s[1] == 2 && g.s[2] == 2 && g.s[3] == 2 && (g.p[1] == 0 || g.p[1] == 1) &&
+                        g.p[2] == 1 && g.p[3] == 1;
+      const bool column = ksel == 2 && g.s[1] == 2 && g.s[2] == 1 && g.s[3] == 1 && g.p[1] == 0 && g.p[2] == 0 && g.p[3] == 0;
+      RbGeom gi = g;
+      for (int dim = 0; dim <= kMaxSpatial; ++dim) gi.shape[dim] = g.inShape[dim];
+      uint64_t inRecords64 = 0;
+      const BlockMap mi = makeBlockMap(gi, &inRecords64);
+      const char* e = debugEnv("D3D_RULEBOOK_GATHER");
+      if ((cube || column) && inRecords64 > 0 && inRecords64 < 0xFFFFFFFFull && !(e && e[0] == '0')) {
+        gather = cube ? 1 : 2;
+        ga.src = RecRef{const_cast<BmRecord*>(static_cast<const BmRecord*>(side.srcRecords)),
+                        side.srcDouble ? side.srcState : nullptr,
+                        side.srcDouble ? static_cast<uint32_t>(side.srcStride) : 0u, 1u};
+        ga.srcChunkBase = side.srcChunkBase;
+        ga.mo = m;
+        ga.mi = mi;
+        ga.numActIn = numActIn;
+        ga.inCap = static_cast<uint32_t>(cap);
+        ga.shapeY = g.shape[3];
+        ga.shapeX = g.shape[4];
+        ga.padZ = g.p[1];
+      }
+    }
+    side.sourceMapUsed = gather != 0;
     if (sharedMap) {
       // the strided build that wrote these coordinates marked and scanned this very grid
+    } else if (gather) {
+      // marked inside the scan
     } else if (subM) {
       hipLaunchKernelGGL(bmMarkInputs, perInput, block, 0, stream, g, m, coors, numActIn, cap, recBefore,
                          needReset ? nullptr : permShuffled);
@@ -2086,13 +2272,19 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       hipLaunchKernelGGL(bmMarkCandidates, perTap, block, 0, stream, g, m, coors, numActIn, cap, recBefore);
     }
     // D3D_RULEBOOK_ORDERED_SCAN=1: acquire-release tickets (see bmScan)
+#define D3D_LAUNCH_SCAN(ORDERED, GATHER)                                                                          \
+  hipLaunchKernelGGL((bmScan<ORDERED, GATHER>), perChunk, dim3(GATHER ? kRbChunk : kRbThreads), 0, stream, recBefore, w.nRecords, chunkBase, \
+                     w.nChunks, scanTicket, scanTicket + 1, subM ? nullptr : numActOut, maxNumActOut, ga)
+    const bool ordered = debugEnv("D3D_RULEBOOK_ORDERED_SCAN") != nullptr;
     if (sharedMap) {
-    } else if (debugEnv("D3D_RULEBOOK_ORDERED_SCAN"))
-      hipLaunchKernelGGL(bmScan<true>, perChunk, block, 0, stream, recBefore, w.nRecords, chunkBase, w.nChunks, scanTicket,
-                         scanTicket + 1, subM ? nullptr : numActOut, maxNumActOut);
-    else
-      hipLaunchKernelGGL(bmScan<false>, perChunk, block, 0, stream, recBefore, w.nRecords, chunkBase, w.nChunks,
-                         scanTicket, scanTicket + 1, subM ? nullptr : numActOut, maxNumActOut);
+    } else if (gather == 1) {
+      if (ordered) D3D_LAUNCH_SCAN(true, 1); else D3D_LAUNCH_SCAN(false, 1);
+    } else if (gather == 2) {
+      if (ordered) D3D_LAUNCH_SCAN(true, 2); else D3D_LAUNCH_SCAN(false, 2);
+    } else {
+      if (ordered) D3D_LAUNCH_SCAN(true, 0); else D3D_LAUNCH_SCAN(false, 0);
+    }
+#undef D3D_LAUNCH_SCAN
     if (!near) {  // the near probe launch carries these passes itself
       if (!subM)
         hipLaunchKernelGGL(bmEmitCoords, dim3(emitBlocks(w.nRecords, kRbThreads)), block, 0, stream,

@@ -88,8 +88,9 @@ class SparseConvLayer:
             ws = torch.empty(max(1, self.idx_plugin.workspace_size(in_descs, out_descs)), dtype=torch.uint8,
                              device=self.device)
             self._idx_state = dict(cap=x.capacity, in_descs=in_descs, out_descs=out_descs, outs=outs, ws=ws)
-            # a SubM rulebook on the outputs of a strided one reuses that operator's occupancy map
-            if self.spec["subm"] and self.extensions:
+            # a SubM rulebook on the outputs of a strided one reuses that operator's occupancy map; a strided one
+            # derives the occupancy of its own map from it
+            if self.extensions and not self.spec.get("inverse", False):
                 self.idx_plugin.link_coords(x.producer)
             self.idx_plugin.configure(in_descs, out_descs)  # reserves the maps an operator keeps between passes
         st = self._idx_state

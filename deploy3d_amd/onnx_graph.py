@@ -367,14 +367,14 @@ class GraphExecutor:
                 continue
             if p.name.startswith("SPConvIdx"):
                 p.set_option(OPT_PERSISTENT_INDEX, 1)  # the executor owns the index tensor and nobody else writes it
-                # a SubM node on the coordinates a strided node wrote reuses that node's occupancy map
+                # a node on the coordinates a strided node wrote works from that node's occupancy map
                 src = producer.get(n.inputs[0])
                 if src is not None and src[1] == 2 and producer.get(n.inputs[1]) == (src[0], 3) and \
                         src[0] in self.plugins and self.plugins[src[0]].name == p.name:
                     try:
                         p.link_coords(self.plugins[src[0]])
                     except EngineError:
-                        pass  # this node is not submanifold
+                        pass
             if p.name == "SPConvMM" and len(n.inputs) >= 5:
                 src = producer.get(n.inputs[3])
                 if src is not None and src[1] == 0 and src[0] in self.plugins and \

@@ -221,8 +221,9 @@ class Plugin:
         _check(self._lib.d3d_link_rulebook(self._h, None if idx_plugin is None else idx_plugin._h))
 
     def link_coords(self, producer):
-        """Submanifold SPConvIdx only: the coordinates it is handed are the output of the strided SPConvIdx
-        ``producer`` (None removes the link), whose occupancy map it then reuses instead of building its own."""
+        """SPConvIdx only: the coordinates it is handed are the output of the strided SPConvIdx ``producer`` (None
+        removes the link).  A submanifold operator then reuses that operator's occupancy map instead of building its
+        own; a strided one derives the occupancy of its output grid from it instead of marking it input by input."""
         _check(self._lib.d3d_link_coords(self._h, None if producer is None else producer._h))
 
     def set_option(self, option, value):

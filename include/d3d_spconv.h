@@ -176,15 +176,18 @@ const char* d3d_op_name(int32_t i);
  * index tensor that names several (duplicate input coordinates) keeps the highest input row. */
 int32_t d3d_link_rulebook(d3d_plugin* mm, d3d_plugin* idx);
 
-/* No counterpart in the reference.  d3d_link_coords(subm, producer) tells the submanifold rulebook operator `subm`
+/* No counterpart in the reference.  d3d_link_coords(consumer, producer) tells the rulebook operator `consumer`
  * that its inCoors / numActIn (inputs 0 and 1) are outCoors / numActOut (outputs 2 and 3) of the strided or
  * transposed operator `producer` - again an edge of the graph.  `producer` then keeps the occupancy map of its
- * output grid in memory the two handles own together (allocated at its next enqueue, freed with the last handle),
- * and `subm` uses it instead of clearing, marking and scanning a map of the same grid itself, whenever the tensors
- * it is handed are the ones `producer` wrote last, on the same grid and capacity; otherwise it builds its own, as
- * an operator nobody linked does.  Several SubM operators may be linked to one producer; producer = NULL removes
- * the link.  As with d3d_link_rulebook: do not link when something edits the coordinates between the two enqueues. */
-int32_t d3d_link_coords(d3d_plugin* subm, d3d_plugin* producer);
+ * output grid in memory the two handles own together (allocated at its next configure or enqueue, freed with the
+ * last handle).  A submanifold `consumer` uses that map instead of clearing, marking and scanning a map of the same
+ * grid itself; a strided one (3x3x3 with stride 2 and padding 1, or 3x1x1 with stride (2,1,1) and padding 0)
+ * derives the occupancy of its own output grid from it instead of marking it input by input - whenever the tensors
+ * it is handed are the ones `producer` wrote last, on the same grid and capacity; otherwise it works from the
+ * coordinates alone, as an operator nobody linked does.  Several operators may be linked to one producer;
+ * producer = NULL removes the link.  As with d3d_link_rulebook: do not link when something edits the coordinates
+ * between the two enqueues. */
+int32_t d3d_link_coords(d3d_plugin* consumer, d3d_plugin* producer);
 
 /* Options, none of which the reference has.
  * D3D_OPT_PERSISTENT_INDEX (SPConvIdx{N}d; value 0 / 1): the caller promises that the index tensor this handle

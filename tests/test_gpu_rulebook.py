@@ -217,6 +217,52 @@ def test_submanifold_on_a_strided_operators_map(engine):
         subm.link_coords(None)
 
 
+@pytest.mark.parametrize("second", [((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((3, 3, 3), (2, 2, 2), (0, 1, 1)),
+                                    ((3, 1, 1), (2, 1, 1), (0, 0, 0)), ((3, 3, 3), (2, 2, 2), (0, 0, 0))])
+def test_strided_operator_on_a_strided_operators_map(engine, second):
+    """d3d_link_coords with a strided consumer: for the kernel shapes it knows it derives the occupancy of its output
+    grid from the producer's map instead of marking it input by input (the last parameter set is a shape it does not
+    know: the link is there and changes nothing).  Odd grid extents (bricks cut by the edge on both levels), two
+    samples, a producer that truncates its outputs (its map then holds cells whose rows were dropped), changing
+    clouds (the producer's two maps take turns); checked against the oracle on the producer's coordinates and
+    against the same operator without the link."""
+    import torch
+    from deploy3d_amd import spconv_index_nd
+    from deploy3d_amd.spconv_index import index_plugin
+    grid, batch, n = (13, 45, 38), 2, 4000
+    rng = np.random.default_rng(123)
+    first = ((3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1), (0, 0, 0))
+    nxt = second + ((1, 1, 1), (0, 0, 0))
+    shape = torch.empty((batch, 0) + grid, dtype=torch.int32, device="cuda")
+    for max1 in (8 * n, 900):
+        max2 = 8 * max1
+        producer = index_plugin(*first, max1, False, False)
+        consumer = index_plugin(*nxt, max2, False, False)
+        for m in (n, 2500, n):
+            coords = random_cloud(rng, m, grid, batch)
+            c = torch.from_numpy(coords).cuda()
+            num = torch.tensor([len(coords)], dtype=torch.int32, device="cuda")
+            canon = []
+            for linked in (True, False):
+                consumer.link_coords(producer if linked else None)
+                _, _, oc, no, osh = spconv_index_nd(c, num, shape, *first, max1, False, False)
+                index, num_index, oc2, no2, osh2 = spconv_index_nd(oc, no, osh, *nxt, max2, False, False)
+                torch.cuda.synchronize()
+                got = oracle.canonical(index.cpu().numpy(), int(num_index.item()), oc2.cpu().numpy(), int(no2.item()))
+                canon.append(got)
+                if linked:
+                    live = int(no.item())
+                    assert live == min(max1, live) and (max1 > 900 or live == 900)
+                    ref = oracle.rulebook(oc.cpu().numpy(), live, (batch,) + tuple(osh2.shape[2:]), *nxt[:4], max2, False)
+                    want = oracle.canonical(ref["index"], ref["num_index"], ref["out_coors"], ref["num_act_out"])
+                    assert int(num_index.item()) == ref["num_index"] and int(no2.item()) == ref["num_act_out"]
+                    np.testing.assert_array_equal(got[0], want[0])
+                    np.testing.assert_array_equal(got[1], want[1])
+            np.testing.assert_array_equal(canon[0][0], canon[1][0])
+            np.testing.assert_array_equal(canon[0][1], canon[1][1])
+        consumer.link_coords(None)
+
+
 def test_ordered_scan_variant(engine, monkeypatch):
     """D3D_RULEBOOK_ORDERED_SCAN=1 selects acquire-release tickets in the scan pass of the block map: same results."""
     monkeypatch.setenv("D3D_RULEBOOK_ORDERED_SCAN", "1")
