@@ -29,9 +29,9 @@ ELEM = {"float16": 2, "bfloat16": 2, "int8": 1, "float32": 4}
 # 256 MiB copy of --pmc-copy-mib (FETCH_SIZE reads half the copied KiB: factor 2.0; WRITE_SIZE factor 1.0).
 # A cached reading: it belongs to the kernel and workload named here and is null for any other.
 TRAFFIC_SOURCE = "profiles/config3_backbone_hbm_traffic_pmc.txt"
-# conv3_0 / conv3_1 run the same kernel on the same rulebook: FETCH_SIZE 46149 and WRITE_SIZE 34539 per dispatch.
-MEASURED_TRAFFIC = {(3, 120000, "conv3_0"): int((46149 * 2.0 + 34539 * 1.0) * 1024),
-                    (3, 120000, "conv3_1"): int((46149 * 2.0 + 34539 * 1.0) * 1024)}
+# conv3_0 / conv3_1 run the same kernel on the same rulebook: FETCH_SIZE 34792 and WRITE_SIZE 34050 per dispatch.
+MEASURED_TRAFFIC = {(3, 120000, "conv3_0"): int((34792 * 2.0 + 34050 * 1.0) * 1024),
+                    (3, 120000, "conv3_1"): int((34792 * 2.0 + 34050 * 1.0) * 1024)}
 DEFAULT_VOXELS = {1: 20000, 2: 60000, 3: 120000, 4: 120000, 5: 250000}
 WORKLOAD = {
     1: "config 1: one SubM 3x3x3 16->16, fp32, %d voxels uniform in grid [41,1600,1408]",
