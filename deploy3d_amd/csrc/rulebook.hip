@@ -1046,7 +1046,17 @@ struct GatherArgs {
   uint32_t inCap;                  // row capacity of the input: a live count below it rules truncation out
   int shapeY, shapeX;              // output extents of the two in-brick dims
   int padZ;                        // GATHER 1: padding of the level dim, 0 or 1
+  float rcpX, rcpY, rcpZ;          // 1 / mo.nb[3], 1 / mo.nb[2], 1 / mo.nb[1] (record indices stay below 2^24)
 };
+
+// x / d for x < 2^24 with rcp = 1.0f / d: the float quotient is off by one at most.
+__device__ __forceinline__ uint32_t divSmall(uint32_t x, uint32_t d, float rcp) {
+  uint32_t q = static_cast<uint32_t>(static_cast<float>(x) * rcp);
+  const int32_t r = static_cast<int32_t>(x - q * d);
+  if (r < 0) --q;
+  else if (r >= static_cast<int32_t>(d)) ++q;
+  return q;
+}
 
 // Cells of an input-map record (bits, rank `first` of its lowest cell) that are rows of the input: cells ranked at
 // or past nLive were cut off when the build that wrote the map truncated its outputs.
@@ -1060,13 +1070,31 @@ __device__ __forceinline__ unsigned long long cutToLive(unsigned long long bits,
   return bits;
 }
 
-// bits 0, 2, .., 14 of x packed into bits 0..7
-__device__ __forceinline__ uint32_t evenBits(uint32_t x) {
-  x &= 0x5555u;
-  x = (x | (x >> 1)) & 0x3333u;
-  x = (x | (x >> 2)) & 0x0F0Fu;
-  x = (x | (x >> 4)) & 0x00FFu;
-  return x;
+// Three consecutive cells OR-ed, every second one kept: with the 8 cells of byte k of `mid` at positions 1..8 of a
+// row of 17, the last cell of byte k of `left` at position 0 and the cells of byte k of `right` at 9..16, byte k
+// of the result holds cell j = OR of positions 2j, 2j+1, 2j+2 - for all 8 bytes at once.
+__device__ __forceinline__ unsigned long long foldCells(unsigned long long left, unsigned long long mid,
+                                                        unsigned long long right) {
+  constexpr unsigned long long k01 = 0x0101010101010101ull;
+  const unsigned long long tm = mid | ((mid >> 1) & (k01 * 0x7F)) | ((mid >> 2) & (k01 * 0x3F));        // bit i: m_i|m_i+1|m_i+2
+  const unsigned long long tr = right | ((right >> 1) & (k01 * 0x7F)) | ((right >> 2) & (k01 * 0x3F));
+  unsigned long long out = (((left >> 7) | mid | (mid >> 1)) & k01);                                     // l7|m0|m1
+  out |= (tm & (k01 * 0x02)) | ((tm >> 1) & (k01 * 0x04)) | ((tm >> 2) & (k01 * 0x08));                  // m1.., m3.., m5..
+  out |= (((mid >> 7) | right | (right >> 1)) & k01) << 4;                                               // m7|r0|r1
+  out |= ((tr & (k01 * 0x02)) << 4) | ((tr & (k01 * 0x08)) << 3) | ((tr & (k01 * 0x20)) << 2);           // r1.., r3.., r5..
+  return out;
+}
+
+// The same fold one level up: rows instead of cells.  `above`, `here`, `below` hold 8 rows of 8 cells each (a byte
+// per row); row k of the result = OR of rows 2k, 2k+1, 2k+2 of the 17 rows (last of above, 8 of here, 8 of below).
+__device__ __forceinline__ unsigned long long foldRows(unsigned long long above, unsigned long long here,
+                                                       unsigned long long below) {
+  const unsigned long long th = here | (here >> 8) | (here >> 16);    // byte i: rows i, i+1, i+2 of here
+  const unsigned long long tb = below | (below >> 8) | (below >> 16);
+  const unsigned long long r0 = ((above >> 56) | here | (here >> 8)) & 0xFFull;
+  const unsigned long long r4 = ((here >> 56) | below | (below >> 8)) & 0xFFull;
+  return r0 | (((th >> 8) & 0xFFull) << 8) | (((th >> 24) & 0xFFull) << 16) | (((th >> 40) & 0xFFull) << 24) |
+         (r4 << 32) | (((tb >> 8) & 0xFFull) << 40) | (((tb >> 24) & 0xFFull) << 48) | (((tb >> 40) & 0xFFull) << 56);
 }
 
 // Occupancy of output record `rec` (a brick of 1 x 8 x 8 cells) from the input map.
@@ -1076,13 +1104,12 @@ __device__ __forceinline__ uint32_t evenBits(uint32_t x) {
 template <int GATHER>
 __device__ __forceinline__ unsigned long long gatherOccupancy(const GatherArgs& ga, const BmRecord* __restrict__ src,
                                                               uint32_t rec, uint32_t nLive, bool checkRanks) {
-  uint32_t q = rec;
-  const int obx = static_cast<int>(q % static_cast<uint32_t>(ga.mo.nb[3]));
-  q /= static_cast<uint32_t>(ga.mo.nb[3]);
-  const int oby = static_cast<int>(q % static_cast<uint32_t>(ga.mo.nb[2]));
-  q /= static_cast<uint32_t>(ga.mo.nb[2]);
-  const int oz = static_cast<int>(q % static_cast<uint32_t>(ga.mo.nb[1]));
-  const uint32_t batch = q / static_cast<uint32_t>(ga.mo.nb[1]);  // the leading spatial dim of a 3-D grid has extent 1
+  const uint32_t q1 = divSmall(rec, static_cast<uint32_t>(ga.mo.nb[3]), ga.rcpX);
+  const int obx = static_cast<int>(rec - q1 * static_cast<uint32_t>(ga.mo.nb[3]));
+  const uint32_t q2 = divSmall(q1, static_cast<uint32_t>(ga.mo.nb[2]), ga.rcpY);
+  const int oby = static_cast<int>(q1 - q2 * static_cast<uint32_t>(ga.mo.nb[2]));
+  const uint32_t batch = divSmall(q2, static_cast<uint32_t>(ga.mo.nb[1]), ga.rcpZ);  // (the leading spatial dim of a 3-D grid has extent 1)
+  const int oz = static_cast<int>(q2 - batch * static_cast<uint32_t>(ga.mo.nb[1]));
   const int nz = ga.mi.nb[1], ny = ga.mi.nb[2], nx = ga.mi.nb[3];
   constexpr int NA = GATHER == 1 ? 3 : 1;           // input bricks under the output brick per in-brick dim
   constexpr int N = 3 * NA * NA;
@@ -1136,22 +1163,9 @@ __device__ __forceinline__ unsigned long long gatherOccupancy(const GatherArgs& 
   if constexpr (GATHER == 2) {
     return under[0][0];
   } else {
-    // input row i of the 17 under the brick (i = 0: the last row of the brick row above) as 17 cells: bit 0 the
-    // last cell of the brick to the left, bits 1..16 the cells of the two bricks underneath
-    auto row17 = [&](int i) -> uint32_t {
-      const int a = i == 0 ? 0 : (i <= 8 ? 1 : 2);
-      const int sh = 8 * (i == 0 ? 7 : (i <= 8 ? i - 1 : i - 9));
-      const uint32_t l = static_cast<uint32_t>(under[a][0] >> sh) & 0xFFu, m = static_cast<uint32_t>(under[a][1] >> sh) & 0xFFu,
-                     r = static_cast<uint32_t>(under[a][2] >> sh) & 0xFFu;
-      return (l >> 7) | (m << 1) | (r << 9);
-    };
-    unsigned long long bits = 0ull;
-#pragma unroll
-    for (int oy = 0; oy < 8; ++oy) {
-      const uint32_t x = row17(2 * oy) | row17(2 * oy + 1) | row17(2 * oy + 2);
-      bits |= static_cast<unsigned long long>(evenBits(x | (x >> 1) | (x >> 2))) << (8 * oy);
-    }
-    return bits;
+    // 17 x 17 input cells under the 8 x 8 outputs: rows folded first (per brick column), then cells
+    return foldCells(foldRows(under[0][0], under[1][0], under[2][0]), foldRows(under[0][1], under[1][1], under[2][1]),
+                     foldRows(under[0][2], under[1][2], under[2][2]));
   }
 }
 
@@ -1187,8 +1201,9 @@ bmScan(RecRef recRef, uint32_t nRecords, uint32_t* chunkBase, uint32_t nChunks, 
       const uint32_t rec = blockIdx.x * kRbChunk + threadIdx.x;
       unsigned long long bits = rec < nRecords ? gatherOccupancy<GATHER>(ga, src, rec, nLive, checkRanks) : 0ull;
       if (bits) {  // cells of the brick past the edge of the output grid are no outputs
-        const int by = static_cast<int>((rec / static_cast<uint32_t>(ga.mo.nb[3])) % static_cast<uint32_t>(ga.mo.nb[2]));
-        const int bx = static_cast<int>(rec % static_cast<uint32_t>(ga.mo.nb[3]));
+        const uint32_t q1 = divSmall(rec, static_cast<uint32_t>(ga.mo.nb[3]), ga.rcpX);
+        const int bx = static_cast<int>(rec - q1 * static_cast<uint32_t>(ga.mo.nb[3]));
+        const int by = static_cast<int>(q1 - divSmall(q1, static_cast<uint32_t>(ga.mo.nb[2]), ga.rcpY) * static_cast<uint32_t>(ga.mo.nb[2]));
         const int rows = ga.shapeY - 8 * by, cols = ga.shapeX - 8 * bx;
         if (rows < 8) bits &= (1ull << (8 * rows)) - 1ull;
         if (cols < 8) bits &= 0x0101010101010101ull * ((1ull << cols) - 1ull);
@@ -2237,7 +2252,8 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
       uint64_t inRecords64 = 0;
       const BlockMap mi = makeBlockMap(gi, &inRecords64);
       const char* e = debugEnv("D3D_RULEBOOK_GATHER");
-      if ((cube || column) && inRecords64 > 0 && inRecords64 < 0xFFFFFFFFull && !(e && e[0] == '0')) {
+      if ((cube || column) && inRecords64 > 0 && inRecords64 < 0xFFFFFFFFull && w.nRecords < (1u << 24) &&
+          !(e && e[0] == '0')) {
         gather = cube ? 1 : 2;
         ga.src = RecRef{const_cast<BmRecord*>(static_cast<const BmRecord*>(side.srcRecords)),
                         side.srcDouble ? side.srcState : nullptr,
@@ -2250,6 +2266,9 @@ int32_t launchRulebook(const RbGeom& g, bool subM, const int32_t* coors, const i
         ga.shapeY = g.shape[3];
         ga.shapeX = g.shape[4];
         ga.padZ = g.p[1];
+        ga.rcpX = 1.0f / static_cast<float>(m.nb[3]);
+        ga.rcpY = 1.0f / static_cast<float>(m.nb[2]);
+        ga.rcpZ = 1.0f / static_cast<float>(m.nb[1]);
       }
     }
     side.sourceMapUsed = gather != 0;
